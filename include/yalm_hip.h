@@ -314,9 +314,15 @@ int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
  * key/value latent, a real-gated linear recurrence, a gated delta rule, softmax attention
  * over cached keys and values with a window or chunk mask) and a feed-forward (none, dense
  * GLU, routed experts with an optional shared expert, a plain two-matrix one), each with
- * its own sizes and constants. Around every sublayer: x += norm_b(f(norm(x))) (pre_norm = 1)
- * or x += norm_b(f(x)) (pre_norm = 0); the norms are rms norms or mean-subtracting layer
- * norms (norm_kind), both with a weight and no bias.
+ * its own sizes and constants. Serial blocks (block_kind = YALM_BLOCK_SERIAL): around every
+ * sublayer x += norm_b(f(norm(x))) (pre_norm = 1) or x += norm_b(f(x)) (pre_norm = 0).
+ * Parallel blocks (YALM_BLOCK_PARALLEL): h = norm1(x), x += ls1 * mixer(h) + ls2 * ff(h), one
+ * norm read by both sublayers, each result scaled elementwise by its own vector. The norms
+ * are rms norms or mean-subtracting layer norms (norm_kind), both with a weight and no bias.
+ * The layer array is the order the layers RUN in: a block of layers that is walked several
+ * times with the same weights is passed unrolled, its entries naming the same tensors, and
+ * every entry has its own caches and states; pre_add is a vector added to the stream before
+ * an entry's opening norm (the per-pass vector of such a loop).
  * One yalm_seq holds ONE sequence: its position, the latent caches and the recurrent
  * and convolution states, all in HBM; yalm_seq_step appends tokens (a whole prompt, a
  * portion of one, or a single decoded token) from where the last call stopped, so the
@@ -328,6 +334,15 @@ int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
 enum { YALM_MIX_LATENT = 0, YALM_MIX_RGLRU = 1, YALM_MIX_DELTA = 2, YALM_MIX_ATTN = 3 };
 enum { YALM_FF_NONE = 0, YALM_FF_DENSE = 1, YALM_FF_MOE = 2, YALM_FF_PLAIN = 3 };
 enum { YALM_NORM_RMS = 0, YALM_NORM_LAYER = 1 };
+enum { YALM_BLOCK_SERIAL = 0, YALM_BLOCK_PARALLEL = 1 };
+/* gated feed-forwards: y = w_down (act(w_gate x) (.) w_up x) */
+enum { YALM_ACT_DEFAULT = 0, /* dense: gelu; experts and shared expert: clamp */
+	   YALM_ACT_GELU = 1,  /* gelu_tanh(g) u */
+	   YALM_ACT_CLAMP = 2, /* g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit) */
+	   YALM_ACT_SILU = 3   /* g sigmoid(g) u */ };
+/* routed experts: how the `top` experts and their weights come from the router logits */
+enum { YALM_ROUTER_SOFTMAX_TOP = 0, /* softmax over all experts, best groups, top scores, weight = score * router_scale */
+	   YALM_ROUTER_TOP_SOFTMAX = 1  /* the top logits (+ router_bias) win, weights = softmax over the chosen logits only */ };
 /* attn: which earlier positions j <= i a position i sees */
 enum { YALM_MASK_CAUSAL = 0, /* all of them */
 	   YALM_MASK_WINDOW = 1, /* i - j < mask_size */
@@ -343,21 +358,30 @@ typedef struct yalm_seq_layer {
 	                                  queries / keys shared by heads / kv_heads value heads of vdim; attn: heads
 	                                  query heads of dim, kv_heads key (dim) / value (vdim) heads, query head h
 	                                  reads key/value head h / (heads / kv_heads) */
-	int kv_rank, q_rank, kv_from;  /* latent: ranks; kv_from >= 0: read that layer's latent cache (no own w_in rows) */
+	int kv_rank, q_rank, kv_from;  /* latent: ranks; kv_from >= 0: read that layer's latent cache (no own w_in rows);
+	                                  q_rank = 0: the queries are projected from the input directly */
+	int rot_dim;                   /* latent with q_rank = 0: every query head is [dim plain | rot_dim rotated] entries and
+	                                  w_in's last rot_dim rows give one rotated key part shared by all heads (not normed),
+	                                  score = (q_plain . W_uk c + q_rot . k_rot) * attn_scale; rotation as rot_dims / rot_base
+	                                  below (rot_dims <= rot_dim); mask_kind / mask_size / sink / sink_w apply */
 	float attn_scale;              /* latent, attn: score = q.k * attn_scale */
 	int rec_width, blocks;         /* rglru: channels, diagonal gate blocks */
 	int conv;                      /* rglru, delta: taps of the causal per-channel convolution */
 	int ff_kind, ff;               /* YALM_FF_*; ff: hidden size (dense, plain) or one expert's (moe) */
 	int experts, top, groups, groups_keep; /* moe: top experts among the groups_keep best of `groups` groups */
-	float router_scale, limit;     /* moe: weight = softmax score * router_scale; expert clamp */
+	float router_scale, limit;     /* moe: weight = softmax score * router_scale; clamp of the dense / expert pair */
 	int shared_ff;                 /* moe: shared expert's hidden size, 0 = none */
 	float shared_limit;
+	int ff_act;                    /* YALM_ACT_*: the gated pair of the dense feed-forward, of the experts and the shared expert */
+	int router_kind;               /* YALM_ROUTER_* */
 	/* attn */
 	int mask_kind, mask_size;      /* YALM_MASK_* and its size in positions */
 	int qk_norm;                   /* YALM_QK_* */
 	int v_norm;                    /* 1: every value head divided by its rms over vdim (no weight) before it is cached */
-	int sink;                      /* 1: the softmax has one more key of score 0 and no value (1 added to the denominator) */
-	int out_gate;                  /* 1: head h's output times sigmoid(w_g[h] . x); the heads gate rows close w_in */
+	int sink;                      /* 1: the softmax has one more key without a value: exp(sink_w[h]) is added to head h's
+	                                  denominator, unscaled (sink_w NULL: score 0, i.e. 1 is added) */
+	int out_gate;                  /* 1: head h's output times sigmoid(w_g[h] . x), heads gate rows close w_in;
+	                                  2: the concatenated heads times sigmoid(W_g x) elementwise, heads vdim gate rows close w_in */
 	int rot_dims, rot_orig;        /* rotary positions on the first rot_dims entries of every query / key head, pairs
 	                                  (2i, 2i + 1), frequency rot_base^(-2i / rot_dims); rot_orig: see rot_factor */
 	float rot_base;
@@ -366,7 +390,12 @@ typedef struct yalm_seq_layer {
 	                                  where slower, f where faster, a linear ramp between), cos and sin times
 	                                  0.1 ln(rot_factor) + 1 */
 	/* f32 vectors */
-	const float *norm1, *norm1b, *norm2, *norm2b; /* [width] each; norm2* unused without a feed-forward */
+	const float *norm1, *norm1b, *norm2, *norm2b; /* [width] each; norm2* unused without a feed-forward; parallel blocks: norm1 only */
+	const float *ls1, *ls2;         /* parallel blocks: [width] scales of the mixer's and the feed-forward's result */
+	const float *pre_add;           /* [width] added to the stream before this entry's opening norm, or NULL */
+	const float *sink_w;            /* [heads], see sink */
+	const float *o_bias;            /* attn: [width] bias of the output projection, or NULL */
+	const float *router_bias;       /* moe: [experts] added to the router logits, or NULL */
 	const float *q_norm, *kv_norm;  /* latent: [q_rank], [kv_rank]; attn with YALM_QK_WHOLE: [heads dim], [kv_heads dim] */
 	const float *in_bias;           /* rglru: [2 rec_width] (gate branch, recurrent branch); attn: [rows of w_in] or NULL */
 	const float *head_temp;         /* attn: [heads], score of head h times head_temp[h], or NULL */
@@ -375,13 +404,14 @@ typedef struct yalm_seq_layer {
 	const float *gate_a, *gate_a_b, *gate_i, *gate_i_b; /* rglru: [blocks][bs][bs], [rec_width] (bs = rec_width / blocks) */
 	const float *lam;               /* rglru: [rec_width] */
 	const float *a_log, *dt_bias, *out_norm; /* delta: [heads], [heads], [vdim] */
-	const float *router, *shared_sg; /* moe: [experts][width], [width] */
+	const float *router, *shared_sg; /* moe: [experts][width]; [width]: the shared expert times sigmoid(shared_sg . x), NULL: times 1 */
 	/* matrices of weight_dtype */
-	const void *w_in;  /* latent: [q_rank (+ kv_rank if own latent)][width] (query down, latent down);
+	const void *w_in;  /* latent: [q_rank (+ kv_rank if own latent)][width] (query down, latent down), with q_rank = 0
+	                      [heads (dim + rot_dim) + kv_rank + rot_dim][width] (queries, latent down, rotated key part);
 	                      rglru: [2 rec_width][width] (gate branch, recurrent branch);
 	                      delta: [2 kv_heads dim + 2 heads vdim + 2 heads][width] (q, k, v, output gate, beta, decay);
-	                      attn: [heads dim + kv_heads dim + kv_heads vdim (+ heads if out_gate)][width] (q, k, v, gate) */
-	const void *w_uq;  /* latent: [heads dim][q_rank] */
+	                      attn: [heads dim + kv_heads dim + kv_heads vdim (+ heads | heads vdim if out_gate)][width] (q, k, v, gate) */
+	const void *w_uq;  /* latent: [heads dim][q_rank] (unused with q_rank = 0) */
 	const void *w_ukt; /* latent: [heads][kv_rank][dim], the key up-projection transposed per head */
 	const void *w_uv;  /* latent: [heads vdim][kv_rank] */
 	const void *w_o;   /* [width][heads vdim | rec_width] */
@@ -391,13 +421,14 @@ typedef struct yalm_seq_layer {
 } yalm_seq_layer;
 
 typedef struct yalm_seq_config {
-	int width, vocab, n_layers, max_tokens; /* max_tokens: positions one sequence may hold */
+	int width, vocab, n_layers, max_tokens; /* n_layers: entries of the layer array (layer runs); max_tokens: positions one sequence may hold */
 	float embed_scale, norm_eps;
 	int weight_dtype; /* YALM_BF16 | YALM_F32 */
 	int norm_kind;    /* YALM_NORM_*: every norm of the model (sublayers, final) */
 	int pre_norm;     /* 1: a sublayer reads norm1 / norm2 of the stream; 0: it reads the stream itself (norm1 / norm2 unused) */
 	int pos_embed;    /* 1: the interleaved sin / cos position vector (frequencies 10000^(-2i / width)) is added to the embedding */
 	float logit_scale; /* logits = head . norm(x) * logit_scale */
+	int block_kind;   /* YALM_BLOCK_*; parallel blocks need pre_norm = 1 */
 } yalm_seq_config;
 
 typedef struct yalm_seq_weights {

@@ -146,7 +146,8 @@ struct E16StoreF32B {
 
 // bf16 operands, the layer-list engine's gated pairs over BRowsGlu rows (gate columns j <
 // FJ / 2, up columns j + FJ / 2 of the same hidden units), C f32: mode 1 gelu_tanh(g) u;
-// mode 2 g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit).
+// mode 2 g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit);
+// mode 3 g sigmoid(g) u.
 struct E16GluB {
 	static constexpr bool NEEDS_LDS = false;
 	static constexpr bool BF16 = true;
@@ -169,6 +170,8 @@ struct E16GluB {
 					float v;
 					if (mode == 1) {
 						v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+					} else if (mode == 3) {
+						v = g / (1.0f + expf(-g)) * u;
 					} else {
 						const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
 						v = gc / (1.0f + expf(-1.702f * gc)) * (uc + 1.0f);

@@ -42,7 +42,7 @@ struct yalm_seq_s {
 	int cap = 0;                 // tokens per internal portion
 	size_t bw = 0;               // floats per row of the work buffers B0..B3
 	int zw = 0;                  // floats per row of Z (the widest input projection)
-	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Z = nullptr, *B[4] = {};
+	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Y2 = nullptr, *Z = nullptr, *B[4] = {};
 	const float *In = nullptr;   // what a sublayer reads: Hn (pre_norm) or X itself
 	float *Xalt = nullptr, *Xbase = nullptr; // single tokens without opening norms: the stream alternates between two rows
 	const float *pend_wb = nullptr; // a closing norm not yet applied: X += norm(Y) pend_wb, owed to the next product
@@ -57,8 +57,8 @@ struct yalm_seq_s {
 	int att_splits = 1;          // key splits of single-token / short-portion attention
 	float *arena = nullptr;      // every recurrent and convolution state of the sequence
 	size_t arena_floats = 0;
-	std::vector<void *> cache;   // per layer: [max_tokens][kv_rank] latent rows (own latent only); attn: key rows
-	std::vector<void *> vcache;  // attn: [max_tokens][kv_heads vdim] value rows
+	std::vector<void *> cache;   // per layer: [max_tokens][kv_rank (+ rot_dim)] latent rows (own latent only); attn: key rows
+	std::vector<void *> vcache;  // attn: [max_tokens][kv_heads vdim] value rows; latent with a rotated key part: the latent rows again
 	std::vector<double *> rot_freq; // attn: [rot_dims / 2] rotary angle per position
 	std::vector<float> rot_mag;
 	std::vector<int> attn_splits; // attn: key splits of single tokens and short portions
@@ -99,23 +99,56 @@ static int cdiv(int a, int b) {
 // ------------------------------------------------------------------ validation
 static int in_rows(const yalm_seq_layer &l) {
 	switch (l.mixer) {
-	case YALM_MIX_LATENT: return l.q_rank + (l.kv_from < 0 ? l.kv_rank : 0);
+	case YALM_MIX_LATENT:
+		if (l.q_rank == 0)
+			return l.heads * (l.dim + l.rot_dim) + l.kv_rank + l.rot_dim;
+		return l.q_rank + (l.kv_from < 0 ? l.kv_rank : 0);
 	case YALM_MIX_RGLRU: return 2 * l.rec_width;
-	case YALM_MIX_ATTN: return l.heads * l.dim + l.kv_heads * (l.dim + l.vdim) + (l.out_gate ? l.heads : 0);
+	case YALM_MIX_ATTN:
+		return l.heads * l.dim + l.kv_heads * (l.dim + l.vdim) +
+		       (l.out_gate == 2 ? l.heads * l.vdim : (l.out_gate ? l.heads : 0));
 	default: return 2 * l.kv_heads * l.dim + 2 * l.heads * l.vdim + 2 * l.heads;
 	}
+}
+
+// latent attention whose queries come from the input directly (q_rank = 0): served by the
+// softmax-attention kernels as one key/value head whose key row is [latent | rotated key part]
+static bool latent_direct(const yalm_seq_layer &l) {
+	return l.mixer == YALM_MIX_LATENT && l.q_rank == 0;
 }
 
 static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> &L) {
 	ARGCHK(c.width > 0 && c.vocab > 0 && c.n_layers > 0 && c.max_tokens > 0, "yalm_seq_create: bad model sizes");
 	ARGCHK(c.weight_dtype == YALM_BF16 || c.weight_dtype == YALM_F32, "yalm_seq_create: weight_dtype must be bf16 or f32");
 	ARGCHK(c.norm_kind == YALM_NORM_RMS || c.norm_kind == YALM_NORM_LAYER, "yalm_seq_create: unknown norm kind");
+	ARGCHK(c.block_kind == YALM_BLOCK_SERIAL || (c.block_kind == YALM_BLOCK_PARALLEL && c.pre_norm),
+	       "yalm_seq_create: blocks are serial, or parallel with pre_norm");
+	const bool par = c.block_kind == YALM_BLOCK_PARALLEL;
 	for (int i = 0; i < c.n_layers; ++i) {
 		const yalm_seq_layer &l = L[i];
 		const std::string at = "yalm_seq_create: layer " + std::to_string(i) + ": ";
-		ARGCHK((l.norm1 || !c.pre_norm) && l.norm1b && l.w_in && l.w_o, at + "missing tensors");
-		if (l.mixer == YALM_MIX_LATENT) {
+		ARGCHK((l.norm1 || !c.pre_norm) && (l.norm1b || par) && l.w_in && l.w_o, at + "missing tensors");
+		ARGCHK(!par || (l.ls1 && (l.ls2 || l.ff_kind == YALM_FF_NONE)), at + "a parallel block needs its scale vectors");
+		ARGCHK(l.ff_act >= YALM_ACT_DEFAULT && l.ff_act <= YALM_ACT_SILU, at + "unknown feed-forward activation");
+		ARGCHK(!l.pre_add || i == 0 || par, at + "a vector added before an entry after the first needs parallel blocks");
+		if (latent_direct(l)) {
+			ARGCHK(l.heads > 0 && l.dim > 0 && l.vdim > 0 && l.kv_rank > 0 && l.rot_dim >= 0 && l.kv_from < 0,
+			       at + "bad latent attention sizes");
+			if ((size_t)l.heads * ((l.kv_rank + 3) / 4) > (size_t)SA_MAX_NA4 * SEQ_THREADS) {
+				set_err(at + "heads x kv_rank above 16384 is not implemented by the attention kernels");
+				return YALM_ERR_UNSUPPORTED;
+			}
+			ARGCHK(l.kv_norm && l.w_ukt && l.w_uv, at + "missing latent attention tensors");
+			ARGCHK(l.mask_kind == YALM_MASK_CAUSAL || ((l.mask_kind == YALM_MASK_WINDOW || l.mask_kind == YALM_MASK_CHUNK) && l.mask_size > 0),
+			       at + "bad attention mask");
+			ARGCHK(l.rot_dims >= 0 && l.rot_dims <= l.rot_dim && l.rot_dims % 2 == 0 && (l.rot_dims == 0 || l.rot_base > 0.0f),
+			       at + "rotary sizes must be even and at most rot_dim");
+			ARGCHK(!(l.rot_factor > 0.0f) || (l.rot_orig > 0 && l.rot_fast > 0.0f && l.rot_slow > 0.0f && l.rot_base != 1.0f),
+			       at + "bad rotary rescaling");
+		} else if (l.mixer == YALM_MIX_LATENT) {
 			ARGCHK(l.heads > 0 && l.dim > 0 && l.vdim > 0 && l.kv_rank > 0 && l.q_rank > 0, at + "bad latent attention sizes");
+			ARGCHK(l.rot_dim == 0 && l.mask_kind == YALM_MASK_CAUSAL && !l.sink,
+			       at + "a rotated key part, a mask or a sink need directly projected queries (q_rank = 0)");
 			if (l.kv_rank > 256) {
 				set_err(at + "kv_rank above 256 is not implemented by the latent attention kernel");
 				return YALM_ERR_UNSUPPORTED;
@@ -153,6 +186,7 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 			       at + "bad attention mask");
 			ARGCHK(l.qk_norm == YALM_QK_NONE || l.qk_norm == YALM_QK_HEAD_UNIT || (l.qk_norm == YALM_QK_WHOLE && l.q_norm && l.kv_norm),
 			       at + "bad query / key norm");
+			ARGCHK(l.out_gate >= 0 && l.out_gate <= 2, at + "unknown output gate");
 			ARGCHK(l.rot_dims >= 0 && l.rot_dims <= l.dim && l.rot_dims % 2 == 0 && (l.rot_dims == 0 || l.rot_base > 0.0f),
 			       at + "rotary sizes must be even and at most dim");
 			ARGCHK(!(l.rot_factor > 0.0f) || (l.rot_orig > 0 && l.rot_fast > 0.0f && l.rot_slow > 0.0f && l.rot_base != 1.0f),
@@ -161,17 +195,19 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 			ARGCHK(false, at + "unknown mixer");
 		}
 		if (l.ff_kind == YALM_FF_DENSE) {
-			ARGCHK(l.ff > 0 && l.w_gate && l.w_up && l.w_down && (l.norm2 || !c.pre_norm) && l.norm2b, at + "bad dense feed-forward");
+			ARGCHK(l.ff > 0 && l.w_gate && l.w_up && l.w_down && (par || ((l.norm2 || !c.pre_norm) && l.norm2b)), at + "bad dense feed-forward");
 		} else if (l.ff_kind == YALM_FF_PLAIN) {
-			ARGCHK(l.ff > 0 && l.w_up && l.w_down && (l.norm2 || !c.pre_norm) && l.norm2b, at + "bad plain feed-forward");
+			ARGCHK(l.ff > 0 && l.w_up && l.w_down && (par || ((l.norm2 || !c.pre_norm) && l.norm2b)), at + "bad plain feed-forward");
 		} else if (l.ff_kind == YALM_FF_MOE) {
 			ARGCHK(l.ff > 0 && l.experts > 0 && l.top > 0 && l.top <= l.experts && l.groups > 0 &&
 			           l.groups <= SEQ_MAX_GROUPS && l.experts % l.groups == 0 && l.groups_keep > 0 &&
 			           l.groups_keep <= l.groups && l.top <= l.groups_keep * (l.experts / l.groups),
 			       at + "bad router sizes");
-			ARGCHK(l.router && l.w_gate && l.w_up && l.w_down && (l.norm2 || !c.pre_norm) && l.norm2b, at + "missing expert tensors");
+			ARGCHK(l.router_kind == YALM_ROUTER_SOFTMAX_TOP || (l.router_kind == YALM_ROUTER_TOP_SOFTMAX && l.groups == 1),
+			       at + "unknown router kind (the top-logits router has no groups)");
+			ARGCHK(l.router && l.w_gate && l.w_up && l.w_down && (par || ((l.norm2 || !c.pre_norm) && l.norm2b)), at + "missing expert tensors");
 			if (l.shared_ff > 0)
-				ARGCHK(l.ws_gate && l.ws_up && l.ws_down && l.shared_sg, at + "missing shared expert tensors");
+				ARGCHK(l.ws_gate && l.ws_up && l.ws_down, at + "missing shared expert tensors");
 		} else {
 			ARGCHK(l.ff_kind == YALM_FF_NONE, at + "unknown feed-forward kind");
 		}
@@ -275,7 +311,7 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	for (const yalm_seq_layer &l : q->L) {
 		zw = std::max(zw, in_rows(l));
 		if (l.mixer == YALM_MIX_LATENT) {
-			bw = std::max({bw, (size_t)l.heads * l.dim, (size_t)l.heads * l.kv_rank, (size_t)l.heads * l.vdim, (size_t)l.q_rank});
+			bw = std::max({bw, (size_t)l.heads * l.dim, (size_t)l.heads * (l.kv_rank + l.rot_dim), (size_t)l.heads * l.vdim, (size_t)l.q_rank});
 		} else if (l.mixer == YALM_MIX_RGLRU) {
 			bw = std::max(bw, (size_t)l.rec_width);
 			arena += (size_t)l.rec_width + (size_t)(l.conv - 1) * l.rec_width;
@@ -302,6 +338,8 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	STRY(sallocT(q, &q->X, cap * c.width));
 	STRY(sallocT(q, &q->Hn, cap * c.width));
 	STRY(sallocT(q, &q->Y, cap * c.width));
+	if (c.block_kind == YALM_BLOCK_PARALLEL)
+		STRY(sallocT(q, &q->Y2, cap * c.width));
 	STRY(sallocT(q, &q->Z, cap * zw));
 	for (int i = 0; i < 4; ++i)
 		STRY(sallocT(q, &q->B[i], cap * bw));
@@ -328,11 +366,12 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 		q->attn_splits.assign(c.n_layers, 1);
 		for (int i = 0; i < c.n_layers; ++i) {
 			const yalm_seq_layer &l = q->L[i];
-			if (l.mixer != YALM_MIX_ATTN)
+			if (l.mixer != YALM_MIX_ATTN && !latent_direct(l))
 				continue;
 			const int span = l.mask_kind == YALM_MASK_CAUSAL ? c.max_tokens : std::min(c.max_tokens, l.mask_size + GEMV_MAX_M);
 			q->attn_splits[i] = std::max(1, std::min(64, cdiv(span, SA_KT)));
-			part = std::max(part, (size_t)GEMV_MAX_M * l.heads * q->attn_splits[i] * (att_rank4(l.vdim) + 4));
+			const int vd = l.mixer == YALM_MIX_ATTN ? l.vdim : l.kv_rank; // the attention's value size
+			part = std::max(part, (size_t)GEMV_MAX_M * l.heads * q->attn_splits[i] * (att_rank4(vd) + 4));
 		}
 		STRY(sallocT(q, &q->att_part, part));
 	}
@@ -365,7 +404,11 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	size_t off = 0;
 	for (int i = 0; i < c.n_layers; ++i) {
 		const yalm_seq_layer &l = q->L[i];
-		if (l.mixer == YALM_MIX_LATENT) {
+		if (latent_direct(l)) {
+			STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * (l.kv_rank + l.rot_dim) * (bf ? 2 : 4)));
+			q->vcache[i] = q->cache[i];
+			STRY(attn_setup(q, i));
+		} else if (l.mixer == YALM_MIX_LATENT) {
 			if (l.kv_from < 0)
 				STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * l.kv_rank * (bf ? 2 : 4)));
 			STRY(bf ? att_attr_ct<uint16_t>(l.kv_rank) : att_attr_ct<float>(l.kv_rank));
@@ -387,7 +430,7 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 		}
 	}
 	for (int i = 0; i < c.n_layers; ++i)
-		if (q->L[i].mixer == YALM_MIX_LATENT && q->L[i].kv_from >= 0)
+		if (q->L[i].mixer == YALM_MIX_LATENT && q->L[i].q_rank > 0 && q->L[i].kv_from >= 0)
 			q->cache[i] = q->cache[q->L[i].kv_from];
 #undef STRY
 	*out = q;
@@ -461,7 +504,7 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 	// plain products of long portions whose shape fits the large-tile GEMM of the prefill unit;
 	// output columns past the last multiple of 128 (a few gate rows closing an input projection)
 	// run on the general kernel as a second, narrow product
-	const bool pair = a.W2 != nullptr && (a.epi == EPI_GLU_GELU || a.epi == EPI_GLU_CLAMP) && !a.bias;
+	const bool pair = a.W2 != nullptr && (a.epi == EPI_GLU_GELU || a.epi == EPI_GLU_CLAMP || a.epi == EPI_GLU_SILU) && !a.bias;
 	const bool single = !a.W2 && (a.epi == EPI_NONE || a.epi == EPI_GELU);
 	const int n_big = pair ? (a.N % 64 == 0 ? a.N : 0) : (single ? a.N & ~127 : 0);
 	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.rows && !a.w_sel && a.z_split == 0 && a.ldw == a.K &&
@@ -472,7 +515,7 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 		HIPCHK(hipGetLastError());
 		const int rc =
 		    pair ? pf_gemm_glu_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, (const uint16_t *)a.W2, a.N, a.C, a.ldc,
-		                            a.epi == EPI_GLU_GELU ? 1 : 2, a.limit, q->stream)
+		                            a.epi == EPI_GLU_GELU ? 1 : (a.epi == EPI_GLU_CLAMP ? 2 : 3), a.limit, q->stream)
 		         : pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, n_big, a.C, a.ldc, a.bias,
 		                        a.epi == EPI_GELU ? 1 : 0, q->stream);
 		if (rc == YALM_OK && n_big < a.N) {
@@ -798,7 +841,9 @@ static int mixer_attn(Seq *q, int li, int n) {
 	const bool bf = c.weight_dtype == YALM_BF16;
 	const int zin = in_rows(l), H = l.heads, V = l.vdim;
 	float *Q = q->B[0], *gate = q->B[1], *ctx = q->B[2];
-	const int zmain = zin - (l.out_gate ? H : 0); // the gate rows are taken by the projection kernel itself
+	// per-head gate rows are taken by the projection kernel itself; elementwise gate rows are
+	// ordinary output columns of the input projection
+	const int zmain = zin - (l.out_gate == 1 ? H : 0);
 	{
 		GemmArgs g = plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zmain, c.width);
 		g.bias = l.in_bias;
@@ -814,7 +859,10 @@ static int mixer_attn(Seq *q, int li, int n) {
 	a.qk_norm = l.qk_norm;
 	a.v_norm = l.v_norm;
 	a.sink = l.sink;
-	a.out_gate = l.out_gate;
+	a.sink_w = l.sink_w;
+	a.KL = l.kv_heads * l.dim;
+	a.VL = l.kv_heads * l.vdim;
+	a.out_gate = l.out_gate == 1;
 	a.rot_dims = l.rot_dims;
 	a.rot_mag = q->rot_mag[li];
 	a.rot_freq = q->rot_freq[li];
@@ -828,9 +876,9 @@ static int mixer_attn(Seq *q, int li, int n) {
 	a.q_mixed = l.talk && n > GEMV_MAX_M ? 1 : 0;
 	const size_t rot_lds = ((size_t)std::max(l.rot_dims, 2) + (a.q_mixed ? (size_t)H * l.dim : 0)) * sizeof(float);
 	// a few tokens: their head jobs spread over several workgroups
-	const int jobs = H + 2 * l.kv_heads + (l.out_gate ? H : 0);
+	const int jobs = H + 2 * l.kv_heads + (a.out_gate ? H : 0);
 	const dim3 pg(n, n <= GEMV_MAX_M ? cdiv(jobs, SEQ_THREADS / 64) : 1);
-	const float *gbias = l.in_bias ? l.in_bias + zmain : nullptr;
+	const float *gbias = l.in_bias && a.out_gate ? l.in_bias + zmain : nullptr;
 	if (bf)
 		seq_attn_prep_kernel<uint16_t><<<pg, SEQ_THREADS, rot_lds, q->stream>>>(
 		    q->Z, zin, a, q->st, Q, (uint16_t *)q->cache[li], (uint16_t *)q->vcache[li], gate, q->In, c.width,
@@ -840,29 +888,111 @@ static int mixer_attn(Seq *q, int li, int n) {
 		    q->Z, zin, a, q->st, Q, (float *)q->cache[li], (float *)q->vcache[li], gate, q->In, c.width,
 		    (const float *)l.w_in + (size_t)zmain * c.width, gbias);
 	HIPCHK(hipGetLastError());
-	const float *gp = l.out_gate ? gate : nullptr;
+	const float *gp = a.out_gate ? gate : nullptr;
 	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, Q, gp, ctx) : attn_core_t<float>(q, li, n, a, Q, gp, ctx));
-	return gemm(q, plain(ctx, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V));
+	if (l.out_gate == 2) {
+		seq_gate_mul_kernel<<<dim3(cdiv(H * V, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(ctx, H * V, q->Z, zin, zin - H * V,
+		                                                                                   H * V);
+		HIPCHK(hipGetLastError());
+	}
+	GemmArgs o = plain(ctx, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V);
+	o.bias = l.o_bias;
+	return gemm(q, o);
+}
+
+// Latent attention with directly projected queries, a rotated key part shared by all heads, a
+// mask and a sink. With k_j = W_uk c_j and v_j = W_uv c_j: q.k_j = (W_uk^T q).c_j and sum_j p_j
+// v_j = W_uv sum_j p_j c_j, so head h attends with the query [W_uk[h]^T q_plain | q_rot] over
+// the cache rows [c_j | k_rot_j] themselves and sums their first kv_rank entries: the softmax-
+// attention kernels with one key/value head, key size kv_rank + rot_dim, value size kv_rank,
+// the value rows aliasing the key rows.
+static int mixer_latent_direct(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const bool bf = c.weight_dtype == YALM_BF16;
+	const int zin = in_rows(l), H = l.heads, D = l.dim, R = l.rot_dim, V = l.vdim, rk = l.kv_rank, KR = rk + R;
+	float *qp = q->B[0], *qa = q->B[1], *ctx = q->B[2], *oh = q->B[3];
+	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
+	const size_t rot_lds = (size_t)std::max(l.rot_dims, 2) * sizeof(float);
+	if (bf)
+		seq_latent_prep_kernel<uint16_t><<<n, SEQ_THREADS, rot_lds, q->stream>>>(
+		    q->Z, zin, H, D, R, rk, l.rot_dims, q->rot_freq[li], l.kv_norm, c.norm_eps, l.attn_scale, q->st, qp, qa,
+		    (uint16_t *)q->cache[li]);
+	else
+		seq_latent_prep_kernel<float><<<n, SEQ_THREADS, rot_lds, q->stream>>>(
+		    q->Z, zin, H, D, R, rk, l.rot_dims, q->rot_freq[li], l.kv_norm, c.norm_eps, l.attn_scale, q->st, qp, qa,
+		    (float *)q->cache[li]);
+	HIPCHK(hipGetLastError());
+	{ // columns [0, kv_rank) of head h's query: W_uk[h]^T q_plain[h], per head [n][dim] x [rank][dim]^T
+		GemmArgs a = plain(qp, H * D, l.w_ukt, D, qa, H * KR, n, rk, D);
+		a.a_bs = D;
+		a.w_bs = (long)rk * D;
+		a.c_bs = KR;
+		TRY(gemm(q, a, H));
+	}
+	AttnArgs a;
+	a.H = H;
+	a.G = 1;
+	a.D = KR;
+	a.V = rk;
+	a.KL = KR;
+	a.VL = KR;
+	a.mask_kind = l.mask_kind;
+	a.mask_size = l.mask_size;
+	a.qk_norm = YALM_QK_NONE;
+	a.v_norm = 0;
+	a.sink = l.sink;
+	a.sink_w = l.sink_w;
+	a.out_gate = 0;
+	a.rot_dims = 0;
+	a.rot_mag = 1.0f;
+	a.rot_freq = nullptr;
+	a.scale = l.attn_scale;
+	a.q_w = a.k_w = a.temp = a.talk = nullptr;
+	a.eps = c.norm_eps;
+	a.q_mixed = 0;
+	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, qa, nullptr, ctx) : attn_core_t<float>(q, li, n, a, qa, nullptr, ctx));
+	{ // o[h] = W_uv[h] ctx[h]
+		GemmArgs b = plain(ctx, H * rk, l.w_uv, rk, oh, H * V, n, V, rk);
+		b.a_bs = rk;
+		b.w_bs = (long)V * rk;
+		b.c_bs = V;
+		TRY(gemm(q, b, H));
+	}
+	GemmArgs o = plain(oh, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V);
+	o.bias = l.o_bias;
+	return gemm(q, o);
 }
 
 // w_down gelu(w_up x)
-static int ff_plain(Seq *q, int li, int n) {
+static int ff_plain(Seq *q, int li, int n, float *out) {
 	const yalm_seq_layer &l = q->L[li];
 	const yalm_seq_config &c = q->c;
 	GemmArgs a = plain(q->In, c.width, l.w_up, c.width, q->B[0], l.ff, n, l.ff, c.width);
 	a.epi = EPI_GELU;
 	TRY(gemm_in(q, a));
-	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, q->Y, c.width, n, c.width, l.ff));
+	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, out, c.width, n, c.width, l.ff));
 }
 
-static int ff_dense(Seq *q, int li, int n) {
+// the epilogue of a gated pair: the layer's ff_act, or the kind's own form
+static int glu_epi(const yalm_seq_layer &l, int dflt) {
+	switch (l.ff_act) {
+	case YALM_ACT_GELU: return EPI_GLU_GELU;
+	case YALM_ACT_CLAMP: return EPI_GLU_CLAMP;
+	case YALM_ACT_SILU: return EPI_GLU_SILU;
+	default: return dflt;
+	}
+}
+
+static int ff_dense(Seq *q, int li, int n, float *out) {
 	const yalm_seq_layer &l = q->L[li];
 	const yalm_seq_config &c = q->c;
 	GemmArgs a = plain(q->In, c.width, l.w_gate, c.width, q->B[0], l.ff, n, l.ff, c.width);
 	a.W2 = l.w_up;
-	a.epi = EPI_GLU_GELU;
+	a.epi = glu_epi(l, EPI_GLU_GELU);
+	a.limit = l.limit;
 	TRY(gemm(q, a));
-	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, q->Y, c.width, n, c.width, l.ff));
+	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, out, c.width, n, c.width, l.ff));
 }
 
 static int ff_moe(Seq *q, int li, int n) {
@@ -873,8 +1003,9 @@ static int ff_moe(Seq *q, int li, int n) {
 	seq_router_kernel<<<n, SEQ_THREADS, (E + l.groups) * sizeof(float), q->stream>>>(q->In, c.width, l.router, E, top, l.groups,
 	                                                                    l.groups_keep, l.router_scale,
 	                                                                    l.shared_ff > 0 ? l.shared_sg : nullptr, q->idx,
-	                                                                    q->wt, q->sgate);
+	                                                                    q->wt, q->sgate, l.router_kind, l.router_bias);
 	HIPCHK(hipGetLastError());
+	const int epi = glu_epi(l, EPI_GLU_CLAMP);
 	if (n <= GEMV_MAX_M) { // one batch per (token, choice): its expert's matrices picked on the device
 		GemmArgs a = plain(q->In, c.width, l.w_gate, c.width, hx, ff, 1, ff, c.width);
 		a.W2 = l.w_up;
@@ -883,7 +1014,7 @@ static int ff_moe(Seq *q, int li, int n) {
 		a.w_sel = q->idx;
 		a.w_bs = (long)ff * c.width;
 		a.c_bs = ff;
-		a.epi = EPI_GLU_CLAMP;
+		a.epi = epi;
 		a.limit = l.limit;
 		TRY(gemm(q, a, slots));
 		GemmArgs b = plain(hx, ff, l.w_down, ff, yx, c.width, 1, c.width, ff);
@@ -904,7 +1035,7 @@ static int ff_moe(Seq *q, int li, int n) {
 		a.rows_bs = q->cap;
 		a.counts = q->counts;
 		a.a_div = top;
-		a.epi = EPI_GLU_CLAMP;
+		a.epi = epi;
 		a.limit = l.limit;
 		TRY(gemm(q, a, E, n));
 		GemmArgs b = plain(hx, ff, l.w_down, ff, yx, c.width, n, c.width, ff);
@@ -917,12 +1048,29 @@ static int ff_moe(Seq *q, int li, int n) {
 	if (l.shared_ff > 0) {
 		GemmArgs a = plain(q->In, c.width, l.ws_gate, c.width, hs, l.shared_ff, n, l.shared_ff, c.width);
 		a.W2 = l.ws_up;
-		a.epi = EPI_GLU_CLAMP;
+		a.epi = epi;
 		a.limit = l.shared_limit;
 		TRY(gemm(q, a));
 		TRY(gemm(q, plain(hs, l.shared_ff, l.ws_down, l.shared_ff, ys, c.width, n, c.width, l.shared_ff)));
 	}
-	return YALM_OK; // the combine of yx (B[1]) and ys (B[3]) happens in the closing norm's launch (add_norm)
+	return YALM_OK; // the combine of yx (B[1]) and ys (B[3]) happens in the closing norm's launch (add_norm, par_close)
+}
+
+// The seam after a parallel block: both sublayers' results join the stream (the experts' combine
+// happens here), the next entry's pre_add and opening norm follow in the same launch.
+static int par_close(Seq *q, int li, int n) {
+	const yalm_seq_config &c = q->c;
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_layer *nx = li + 1 < c.n_layers ? &q->L[li + 1] : nullptr;
+	const bool moe = l.ff_kind == YALM_FF_MOE;
+	const bool gated = moe && l.shared_ff > 0 && l.shared_sg;
+	float *dump = q->dump_on && q->dump ? q->dump + (size_t)li * n * c.width : nullptr;
+	seq_par_close_kernel<<<n, SEQ_THREADS, (size_t)c.width * sizeof(float), q->stream>>>(
+	    q->X, q->Y, l.ls1, (l.ff_kind != YALM_FF_NONE && !moe) ? q->Y2 : nullptr, l.ls2, moe ? q->B[1] : nullptr, q->wt,
+	    moe ? l.top : 0, moe && l.shared_ff > 0 ? q->B[3] : nullptr, gated ? q->sgate : nullptr, dump,
+	    nx ? nx->pre_add : nullptr, c.norm_eps, c.width, nx ? nx->norm1 : nullptr, q->Hn, (int)q->ln);
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
 }
 
 // moe: the layer's routed experts feed the norm (their combine happens inside it) instead of Y
@@ -968,18 +1116,21 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	if (c.weight_dtype == YALM_F32)
 		seq_embed_kernel<WF32><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
 		                                                         c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
-		                                                         q->Hn, (int)q->ln);
+		                                                         q->Hn, (int)q->ln, q->L[0].pre_add);
 	else
 		seq_embed_kernel<WBF16><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
 		                                                          c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
-		                                                          q->Hn, (int)q->ln);
+		                                                          q->Hn, (int)q->ln, q->L[0].pre_add);
 	HIPCHK(hipGetLastError());
+	const bool par = c.block_kind == YALM_BLOCK_PARALLEL;
 	for (int li = 0; li < c.n_layers; ++li) {
 		const yalm_seq_layer &l = q->L[li];
 		const float *next = pre && li + 1 < c.n_layers ? q->L[li + 1].norm1 : nullptr;
 		if (l.mixer != YALM_MIX_ATTN)
 			TRY(flush_norm(q, n)); // only the attention mixer's input projection takes an owed norm
-		if (l.mixer == YALM_MIX_LATENT)
+		if (latent_direct(l))
+			TRY(mixer_latent_direct(q, li, n));
+		else if (l.mixer == YALM_MIX_LATENT)
 			TRY(mixer_latent(q, li, n));
 		else if (l.mixer == YALM_MIX_RGLRU)
 			TRY(mixer_rglru(q, li, n));
@@ -987,14 +1138,24 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 			TRY(mixer_attn(q, li, n));
 		else
 			TRY(mixer_delta(q, li, n));
+		if (par) { // both sublayers read Hn; the feed-forward's result goes beside the mixer's
+			if (l.ff_kind == YALM_FF_DENSE)
+				TRY(ff_dense(q, li, n, q->Y2));
+			else if (l.ff_kind == YALM_FF_PLAIN)
+				TRY(ff_plain(q, li, n, q->Y2));
+			else if (l.ff_kind == YALM_FF_MOE)
+				TRY(ff_moe(q, li, n));
+			TRY(par_close(q, li, n));
+			continue;
+		}
 		if (l.ff_kind == YALM_FF_NONE) {
 			TRY(close(l.norm1b, next, nullptr));
 		} else {
 			TRY(close(l.norm1b, pre ? l.norm2 : nullptr, nullptr));
 			if (l.ff_kind != YALM_FF_PLAIN)
 				TRY(flush_norm(q, n));
-			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n)
-			                               : (l.ff_kind == YALM_FF_PLAIN ? ff_plain(q, li, n) : ff_moe(q, li, n)));
+			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n, q->Y)
+			                               : (l.ff_kind == YALM_FF_PLAIN ? ff_plain(q, li, n, q->Y) : ff_moe(q, li, n)));
 			TRY(close(l.norm2b, next, l.ff_kind == YALM_FF_MOE ? &l : nullptr));
 		}
 		if (q->dump_on && q->dump)

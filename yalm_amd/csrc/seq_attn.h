@@ -34,7 +34,15 @@ struct AttnArgs {
 	const float *talk;        // [H][H] or null
 	float eps;
 	int q_mixed;              // talk: the projection kernel has already written the mixed queries [t][H][G D]
+	int KL = 0, VL = 0;       // entries per key / value cache row (head g's keys at column g D, values at g V)
+	const float *sink_w = nullptr; // sink: [H] scores of the valueless key, unscaled; null: 0
 };
+
+// The softmax's starting state for head h: with a sink, a valueless key of score sink_w[h] (or 0)
+// has already been seen (running maximum = its score, running sum 1).
+__device__ __forceinline__ float attn_sink_score(const AttnArgs &a, int h) {
+	return a.sink_w ? a.sink_w[h] : 0.0f;
+}
 
 // First key position that position p sees.
 __host__ __device__ __forceinline__ int attn_first_key(int mask_kind, int mask_size, int p) {
@@ -232,6 +240,70 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 	}
 }
 
+// ------------------------------------------------------------------ latent attention with a rotated key part
+// Token t (blockIdx.x) at position p = st->pos + t. Z row: [q: H heads of (D plain | R rotated)
+// | latent: rank | rotated key part: R] (the input projection's result). The latent is rms-
+// normed with weight kv_w into columns [0, rank) of cache row p, the key part is rotated into
+// columns [rank, rank + R) (not normed); every head's plain query part leaves scaled in
+// Qp [t][H][D] (the operand of the per-head product with the transposed key up-projection,
+// which fills columns [0, rank) of Qa) and its rotated part, rotated and scaled, in columns
+// [rank, rank + R) of Qa [t][H][rank + R]: the attention kernels then see H independent heads
+// over ONE key/value head whose key row is the cache row and whose value is its first rank
+// entries. Rotation: the first rot_dims <= R entries in interleaved pairs, as in
+// seq_attn_prep_kernel. Dynamic LDS: max(rot_dims, 2) floats.
+template <class CT>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const float *__restrict__ Z, int ldz, int H, int D,
+                                                                      int R, int rank, int rot_dims,
+                                                                      const double *__restrict__ rot_freq,
+                                                                      const float *__restrict__ kv_w, float eps,
+                                                                      float scale, const StepState *__restrict__ st,
+                                                                      float *__restrict__ Qp, float *__restrict__ Qa,
+                                                                      CT *__restrict__ cache) {
+	extern __shared__ float rot[];
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x, tid = threadIdx.x;
+	const int p = st->pos + t;
+	const int half = rot_dims >> 1;
+	for (int i = tid; i < half; i += SEQ_THREADS) {
+		const double two_pi = 6.283185307179586476925286766559;
+		const double ang = (double)p * rot_freq[i];
+		const float red_ang = (float)(ang - two_pi * rint(ang * (1.0 / two_pi)));
+		rot[i] = cosf(red_ang);
+		rot[half + i] = sinf(red_ang);
+	}
+	const int QH = D + R, QN = H * QH, KR = rank + R;
+	const float *z = Z + (size_t)t * ldz;
+	const float *lat = z + QN;
+	float ss = 0.0f;
+	for (int i = tid; i < rank; i += SEQ_THREADS)
+		ss = fmaf(lat[i], lat[i], ss);
+	const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)rank + eps); // also orders rot[] before its readers
+	CT *crow = cache + (size_t)p * KR;
+	for (int i = tid; i < rank; i += SEQ_THREADS)
+		cache_store<CT>(crow + i, lat[i] * r * kv_w[i]);
+	// the rotated parts: job 0 is the shared key part, job 1 + h head h's query part
+	for (int i = tid; i < (H + 1) * R; i += SEQ_THREADS) {
+		const int job = i / R, d = i - job * R;
+		const float *src = job == 0 ? lat + rank : z + (size_t)(job - 1) * QH + D;
+		float v;
+		if (d < rot_dims) {
+			const float u = src[d & ~1], w = src[d | 1];
+			const float c = rot[d >> 1], sn = rot[half + (d >> 1)];
+			v = (d & 1) ? w * c + u * sn : u * c - w * sn;
+		} else {
+			v = src[d];
+		}
+		if (job == 0)
+			cache_store<CT>(crow + rank + d, v);
+		else
+			Qa[((size_t)t * H + job - 1) * KR + rank + d] = v * scale;
+	}
+	for (int i = tid; i < H * D; i += SEQ_THREADS) {
+		const int h = i / D, d = i - h * D;
+		Qp[(size_t)t * H * D + i] = z[(size_t)h * QH + d] * scale;
+	}
+}
+
 // ------------------------------------------------------------------ attention, f32 FMA form
 // A workgroup owns TQ tokens x the Hb = H / G heads of one key/value head (gridDim.z = G; rows
 // r = tq Hb + hl) and walks its share of the keys they see in tiles of SA_KT. Without score
@@ -337,7 +409,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 	const bool sink0 = a.sink && split == 0;
 	for (int r = tid; r < R; r += SEQ_THREADS) {
 		const int t = t0 + r / Hb;
-		mrun[r] = sink0 ? 0.0f : -FLT_MAX;
+		mrun[r] = sink0 ? attn_sink_score(a, h0 + r % Hb) : -FLT_MAX;
 		lrun[r] = sink0 ? 1.0f : 0.0f;
 		alpha[r] = 1.0f;
 		rlo[r] = t < n_tok ? attn_first_key(a.mask_kind, a.mask_size, pos0 + t) : 0x7fffffff;
@@ -353,7 +425,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 		// ---- scores
 		for (int c = 0; c < Gb; ++c) {
 			__syncthreads(); // the previous readers of cs are done
-			sa_fill_tile<CT>(cs, ldk, Kc, G * D, (g0 + c) * D, D, kt, k_end);
+			sa_fill_tile<CT>(cs, ldk, Kc, a.KL, (g0 + c) * D, D, kt, k_end);
 			__syncthreads();
 			const float4_t *cj = (const float4_t *)(cs + lane * ldk);
 			for (int i0 = wave * rg; i0 < R; i0 += rg * (SEQ_THREADS / 64)) {
@@ -415,7 +487,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 		// ---- weighted sums of the values
 		{
 			__syncthreads(); // the weights are written / the previous readers of cs are done
-			sa_fill_tile<CT>(cs, ldk, Vc, G * V, vg * V, V, kt, k_end);
+			sa_fill_tile<CT>(cs, ldk, Vc, a.VL, vg * V, V, kt, k_end);
 			__syncthreads();
 #pragma unroll
 			for (int x = 0; x < NA4; ++x) {
@@ -498,7 +570,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const floa
 	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
 	const bool talk = a.talk != nullptr;
 	const int Hb = rep, h0 = blockIdx.y * rep; // the heads of one key/value head
-	const int DK = talk ? G * D : D, KL = G * D, VL = G * V, kcol = talk ? 0 : blockIdx.y * D;
+	const int DK = talk ? G * D : D, KL = a.KL, VL = a.VL, kcol = talk ? 0 : blockIdx.y * D;
 	const int DK8 = (DK + 7) & ~7, V4n = (V + 3) >> 2;
 	float *qs = lds;               // [Hb][DK8]
 	float *ps = qs + Hb * DK8;     // [Hb][SA_KT] softmax weights
@@ -541,7 +613,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const floa
 	}
 	const bool sink0 = a.sink && split == 0;
 	for (int r = tid; r < Hb; r += SEQ_THREADS) {
-		mrun[r] = sink0 ? 0.0f : -FLT_MAX;
+		mrun[r] = sink0 ? attn_sink_score(a, h0 + r) : -FLT_MAX;
 		lrun[r] = sink0 ? 1.0f : 0.0f;
 		alpha[r] = 1.0f;
 	}
@@ -753,7 +825,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 	const int lr = lane & 15, lq = lane >> 4;
 	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
 	const bool talk = a.talk != nullptr;
-	const int DK = talk ? G * D : D, KL = G * D, VL = G * V;
+	const int DK = talk ? G * D : D, KL = a.KL, VL = a.VL;
 	const int g = blockIdx.y;
 	const int kcol = talk ? 0 : g * D;
 	const int TB = 4 / HW, tb = wave / HW, hl = blockIdx.z * HW + wave % HW;
@@ -796,7 +868,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 		const bool ok = wave_on && t < n_tok;
 		lo_[r] = ok ? attn_first_key(a.mask_kind, a.mask_size, pos0 + t) : 0x7fffffff;
 		hi_[r] = ok ? pos0 + t : -1;
-		mrun[r] = a.sink ? 0.0f : -FLT_MAX;
+		mrun[r] = a.sink ? attn_sink_score(a, h) : -FLT_MAX;
 		lrun[r] = a.sink ? 1.0f : 0.0f;
 	}
 	f32x4a_t oacc[NT];

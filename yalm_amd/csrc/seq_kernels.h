@@ -65,7 +65,8 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 
 // ------------------------------------------------------------------ embedding
 // X[t] = embed[token] * scale (+ the interleaved (sin, cos) position vector of position
-// st->pos + t if inv_freq); tokens == nullptr: the single device-resident token of the greedy
+// st->pos + t if inv_freq) (+ pre_add, a vector the first layer adds to the stream before its
+// opening norm); tokens == nullptr: the single device-resident token of the greedy
 // loop. w_next != nullptr: also Hn[t] = norm(X[t]) * w_next, the first layer's opening norm.
 template <class WT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState *__restrict__ st,
@@ -74,7 +75,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
                                                                 const float *__restrict__ inv_freq, int width,
                                                                 int vocab, float scale, float *__restrict__ X,
                                                                 const float *__restrict__ w_next, float eps,
-                                                                float *__restrict__ Hn, int ln) {
+                                                                float *__restrict__ Hn, int ln,
+                                                                const float *__restrict__ pre_add = nullptr) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	int tok = tokens ? tokens[t] : st->token;
@@ -87,7 +89,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
 			const float ang = p * inv_freq[i >> 1];
 			pe = (i & 1) ? cosf(ang) : sinf(ang);
 		}
-		const float v = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
+		float v = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
+		if (pre_add)
+			v += pre_add[i];
 		X[(size_t)t * width + i] = v;
 		ss = fmaf(v, v, ss);
 		sm += v;
@@ -319,8 +323,81 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__rest
 		Hn[(size_t)t * n + i] = (row[i] - mu2) * r2 * w_next[i];
 }
 
+// The seam after a parallel block, one launch: X[t] += s1 * Y1[t] + s2 * Y2[t] (s1, s2 the
+// block's elementwise scales; Y2 == nullptr and Yx == nullptr: no feed-forward). Yx != nullptr:
+// the feed-forward's row is the routed experts' combine sum_k wt[t][k] Yx[t top + k] (+ sgate[t]
+// Ys[t], the shared expert; sgate == nullptr: + Ys[t]), summed in slot order. dump != nullptr:
+// the row after the sums is also written there (the stream as the block leaves it). Then
+// X[t] += add (the vector the next layer adds before its opening norm) and, if w_next, Hn[t]
+// = norm(X[t]) * w_next. Dynamic LDS: n floats.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__restrict__ X, const float *__restrict__ Y1,
+                                                                    const float *__restrict__ s1,
+                                                                    const float *__restrict__ Y2,
+                                                                    const float *__restrict__ s2,
+                                                                    const float *__restrict__ Yx,
+                                                                    const float *__restrict__ wt, int top,
+                                                                    const float *__restrict__ Ys,
+                                                                    const float *__restrict__ sgate,
+                                                                    float *__restrict__ dump,
+                                                                    const float *__restrict__ add, float eps, int n,
+                                                                    const float *__restrict__ w_next,
+                                                                    float *__restrict__ Hn, int ln) {
+	extern __shared__ float row[];
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x;
+	float *x = X + (size_t)t * n;
+	float ss = 0.0f, sm = 0.0f;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		float v = fmaf(s1[i], Y1[(size_t)t * n + i], x[i]);
+		if (Yx) {
+			float f = 0.0f;
+			for (int k = 0; k < top; ++k)
+				f = fmaf(wt[(size_t)t * top + k], Yx[((size_t)t * top + k) * n + i], f);
+			if (Ys)
+				f = fmaf(sgate ? sgate[t] : 1.0f, Ys[(size_t)t * n + i], f);
+			v = fmaf(s2[i], f, v);
+		} else if (Y2) {
+			v = fmaf(s2[i], Y2[(size_t)t * n + i], v);
+		}
+		if (dump)
+			dump[(size_t)t * n + i] = v;
+		if (add)
+			v += add[i];
+		x[i] = v;
+		row[i] = v;
+		ss = fmaf(v, v, ss);
+		sm += v;
+	}
+	if (!w_next)
+		return;
+	float mu = 0.0f;
+	if (ln) { // each thread re-reads the entries it wrote
+		mu = block_sum(sm, red) / (float)n;
+		ss = 0.0f;
+		for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+			const float d = row[i] - mu;
+			ss = fmaf(d, d, ss);
+		}
+	}
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
+		Hn[(size_t)t * n + i] = (row[i] - mu) * r * w_next[i];
+}
+
+// C[t][j] *= sigmoid(Z[t][col0 + j]), j < n: an elementwise output gate whose logits are
+// columns of the input projection's result.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_gate_mul_kernel(float *__restrict__ C, int ldc,
+                                                                   const float *__restrict__ Z, int ldz, int col0,
+                                                                   int n) {
+	const int t = blockIdx.y;
+	const int j = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (j < n)
+		C[(size_t)t * ldc + j] *= sq_sigmoid(Z[(size_t)t * ldz + col0 + j]);
+}
+
 // ------------------------------------------------------------------ matrix products
-enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3, EPI_GELU = 4 };
+enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3, EPI_GELU = 4, EPI_GLU_SILU = 5 };
 
 // C[c_row(m)][n] = epi(sum_k A[a_row(m)][k] W[n][k]) for every batch z = blockIdx.z.
 struct GemmArgs {
@@ -361,6 +438,7 @@ __device__ __forceinline__ float epi_apply(const GemmArgs &a, float v, float v2,
 		const float u = fminf(fmaxf(v2, -a.limit), a.limit);
 		return g * sq_sigmoid(1.702f * g) * (u + 1.0f);
 	}
+	case EPI_GLU_SILU: return sq_silu(v) * v2;
 	case EPI_SIGMOID: return sq_sigmoid(v + b);
 	case EPI_GELU: return sq_gelu_tanh(v + b);
 	default: return v + b;
@@ -1657,16 +1735,19 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_mfma_kernel(const
 }
 
 // ------------------------------------------------------------------ routed experts
-// One workgroup per token: router logits in f32, softmax over all experts, a group's score
-// = its best expert's, only experts of the `keep` best groups can be chosen, the `top`
-// largest scores among them win (ties: the lower index); weight = score * rscale, not
-// renormalised. Also the shared expert's gate sigmoid(w_sg . h). Dynamic LDS: E + G floats.
+// One workgroup per token: router logits (+ bias) in f32. kind 0: softmax over all experts, a
+// group's score = its best expert's, only experts of the `keep` best groups can be chosen, the
+// `top` largest scores among them win (ties: the lower index); weight = score * rscale, not
+// renormalised. kind 1: the `top` largest logits win (ties: the lower index), weights =
+// softmax over the chosen logits only. Also the shared expert's gate sigmoid(w_sg . h).
+// Dynamic LDS: E + G floats.
 #define SEQ_MAX_GROUPS 64
 __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__restrict__ Hn, int width,
                                                                  const float *__restrict__ Wr, int E, int top, int G,
                                                                  int keep, float rscale,
                                                                  const float *__restrict__ w_sg, int *__restrict__ idx,
-                                                                 float *__restrict__ wt, float *__restrict__ sgate) {
+                                                                 float *__restrict__ wt, float *__restrict__ sgate,
+                                                                 int kind = 0, const float *__restrict__ bias = nullptr) {
 	extern __shared__ float sc[];
 	const int t = blockIdx.x;
 	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -1692,12 +1773,36 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__
 		a = wave_sum(a);
 		if (lane == 0) {
 			if (e < E)
-				sc[e] = a;
+				sc[e] = a + (bias ? bias[e] : 0.0f);
 			else
 				sgate[t] = sq_sigmoid(a);
 		}
 	}
 	__syncthreads();
+	if (kind == 1) {
+		if (threadIdx.x != 0)
+			return;
+		float zmax = 0.0f, sum = 0.0f;
+		for (int k = 0; k < top; ++k) {
+			int best = 0;
+			float bv = -INFINITY; // finite logits: a taken expert (-inf) never wins
+			for (int e = 0; e < E; ++e)
+				if (sc[e] > bv) {
+					bv = sc[e];
+					best = e;
+				}
+			if (k == 0)
+				zmax = bv;
+			const float w = expf(bv - zmax);
+			idx[(size_t)t * top + k] = best;
+			wt[(size_t)t * top + k] = w;
+			sum += w;
+			sc[best] = -INFINITY;
+		}
+		for (int k = 0; k < top; ++k)
+			wt[(size_t)t * top + k] /= sum;
+		return;
+	}
 	float *gsc = sc + E; // [G]
 	__shared__ float red[SEQ_THREADS / 64];
 	float mx = -FLT_MAX;

@@ -5,8 +5,10 @@ A layer-list design gives every layer its own token mixer and feed-forward
 description; a design registers a reader that turns its ``config.json`` into one and
 a packer that turns its checkpoint tensors into the engine's per-layer tensors
 (concatenated input projections, per-head transposed key up-projections, stacked
-experts). ``Sinulorn`` (latent attention, recurrences, routed experts) and ``Lenuzen``
-(windowed / chunked softmax attention, plain feed-forwards) are such designs.
+experts). ``Sinulorn`` (latent attention, recurrences, routed experts), ``Lenuzen``
+(windowed / chunked softmax attention, plain feed-forwards) and ``Mirorax`` (parallel
+blocks with layer scales, a looped run of layers, gated attention, latent attention with a
+rotated key part, a window and a learned sink) are such designs.
 
 Checkpoints are folders with ``config.json`` and ``model.safetensors`` (bf16
 matrices; read with yalmfile.read_yalm, the same container the .yalm files use).
@@ -27,6 +29,10 @@ FF_NONE, FF_DENSE, FF_MOE, FF_PLAIN = 0, 1, 2, 3
 NORM_RMS, NORM_LAYER = 0, 1
 MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
 QK_NONE, QK_HEAD_UNIT, QK_WHOLE = 0, 1, 2
+BLOCK_SERIAL, BLOCK_PARALLEL = 0, 1
+ACT_DEFAULT, ACT_GELU, ACT_CLAMP, ACT_SILU = 0, 1, 2, 3
+ROUTER_SOFTMAX_TOP, ROUTER_TOP_SOFTMAX = 0, 1
+GATE_NONE, GATE_HEAD, GATE_ELEMENT = 0, 1, 2
 
 
 @dataclasses.dataclass
@@ -69,16 +75,32 @@ class LayerSpec:
     in_biased: bool = False
     head_temps: bool = False
     talking: bool = False
+    # latent attention with directly projected queries (q_rank 0): the rotated part of a
+    # query head and of the one key part all heads share
+    rot_dim: int = 0
+    sink_learned: bool = False  # the sink's score is a tensor (sink_w) instead of 0
+    o_biased: bool = False
+    # gated feed-forwards and routers
+    ff_act: int = ACT_DEFAULT
+    router_kind: int = ROUTER_SOFTMAX_TOP
+    router_biased: bool = False
+    shared_gated: bool = True   # the shared expert is scaled by sigmoid(shared_sg . x)
+    # layer runs
+    pre_added: bool = False     # a vector joins the stream before this run's opening norm
+    shares: int = -1            # >= 0: this run uses the tensors of that (earlier) run, all but pre_add
 
     @property
     def in_rows(self) -> int:
         """Rows of the concatenated input projection w_in."""
         if self.mixer == MIX_LATENT:
+            if self.q_rank == 0:
+                return self.heads * (self.dim + self.rot_dim) + self.kv_rank + self.rot_dim
             return self.q_rank + (self.kv_rank if self.kv_from < 0 else 0)
         if self.mixer == MIX_RGLRU:
             return 2 * self.rec_width
         if self.mixer == MIX_ATTN:
-            return self.heads * self.dim + self.kv_heads * (self.dim + self.vdim) + (self.heads if self.out_gate else 0)
+            gate = {GATE_NONE: 0, GATE_HEAD: self.heads, GATE_ELEMENT: self.heads * self.vdim}[self.out_gate]
+            return self.heads * self.dim + self.kv_heads * (self.dim + self.vdim) + gate
         return 2 * self.kv_heads * self.dim + 2 * self.heads * self.vdim + 2 * self.heads
 
     @property
@@ -102,6 +124,7 @@ class LayeredConfig:
     pos_embed: bool = True    # the sin / cos position vector added to the embedding
     logit_scale: float = 1.0
     tied_head: bool = False   # the logits read the embedding table
+    block_kind: int = BLOCK_SERIAL  # BLOCK_PARALLEL: x += ls1 * mixer(norm1(x)) + ls2 * ff(norm1(x))
 
     def with_(self, **kw) -> "LayeredConfig":
         return dataclasses.replace(self, **kw)
@@ -111,20 +134,35 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
     """field -> (shape, kind) of one layer's engine tensors; kind "w": a matrix of the
     model's weight dtype, "f": f32."""
     W = c.width
-    out = {"norm1b": ((W,), "f")}
-    if c.pre_norm:
-        out["norm1"] = ((W,), "f")
-    if l.ff_kind != FF_NONE:
-        out["norm2b"] = ((W,), "f")
+    out = {}
+    if l.pre_added:
+        out["pre_add"] = ((W,), "f")
+    if l.shares >= 0:
+        return out
+    if c.block_kind == BLOCK_PARALLEL:
+        out["norm1"] = out["ls1"] = ((W,), "f")
+        if l.ff_kind != FF_NONE:
+            out["ls2"] = ((W,), "f")
+    else:
+        out["norm1b"] = ((W,), "f")
         if c.pre_norm:
-            out["norm2"] = ((W,), "f")
+            out["norm1"] = ((W,), "f")
+        if l.ff_kind != FF_NONE:
+            out["norm2b"] = ((W,), "f")
+            if c.pre_norm:
+                out["norm2"] = ((W,), "f")
     out["w_in"] = ((l.in_rows, W), "w")
     out["w_o"] = ((W, l.mix_out), "w")
+    if l.o_biased:
+        out["o_bias"] = ((W,), "f")
+    if l.sink_learned:
+        out["sink_w"] = ((l.heads,), "f")
     if l.mixer == MIX_LATENT:
-        out["q_norm"] = ((l.q_rank,), "f")
+        if l.q_rank:
+            out["q_norm"] = ((l.q_rank,), "f")
+            out["w_uq"] = ((l.heads * l.dim, l.q_rank), "w")
         if l.kv_from < 0:
             out["kv_norm"] = ((l.kv_rank,), "f")
-        out["w_uq"] = ((l.heads * l.dim, l.q_rank), "w")
         out["w_ukt"] = ((l.heads, l.kv_rank, l.dim), "w")
         out["w_uv"] = ((l.heads * l.vdim, l.kv_rank), "w")
     elif l.mixer == MIX_RGLRU:
@@ -154,9 +192,13 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
     elif l.ff_kind == FF_MOE:
         out.update(router=((l.experts, W), "f"), w_gate=((l.experts, l.ff, W), "w"),
                    w_up=((l.experts, l.ff, W), "w"), w_down=((l.experts, W, l.ff), "w"))
+        if l.router_biased:
+            out["router_bias"] = ((l.experts,), "f")
         if l.shared_ff:
-            out.update(shared_sg=((W,), "f"), ws_gate=((l.shared_ff, W), "w"), ws_up=((l.shared_ff, W), "w"),
+            out.update(ws_gate=((l.shared_ff, W), "w"), ws_up=((l.shared_ff, W), "w"),
                        ws_down=((W, l.shared_ff), "w"))
+            if l.shared_gated:
+                out["shared_sg"] = ((W,), "f")
     return out
 
 
@@ -502,9 +544,214 @@ def lenuzen_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0) -> dict:
     return out
 
 
+# ------------------------------------------------------------------ Mirorax
+# Every layer is a parallel block: h = rms(x) w1, x += ls1 * mixer(h) + ls2 * ff(h). A run of
+# layers [start, stop) is walked `times` times with the same weights; pass t first adds row t of
+# the tensor loop.step to the stream; every pass has caches of its own. Two mixers:
+#   "attention":        grouped key/value heads, biased q / k / v / o projections, no positions,
+#                       causal, plain softmax, the concatenated heads times sigmoid(W_g h);
+#   "latent_attention": queries [dim plain | rot_dim rotated] per head from the input directly,
+#                       a cached rms-normed latent (per-head plain keys and values are its
+#                       up-projections) and one cached rotated key part shared by all heads,
+#                       a sliding window, a learned per-head sink in the softmax's denominator.
+# Feed-forwards: "dense" W_d (g' sigmoid(1.702 g') (u' + 1)) with g' = min(W_g h, limit), u' =
+# clamp(W_u h, +-limit); "moe": silu-gated experts, the top logits of a biased router win and
+# their weights are the softmax over the chosen logits, plus an ungated shared expert.
+MIRORAX_MIXERS = ("attention", "latent_attention")
+
+
+def unroll_loop(layers: list, loop) -> list:
+    """The order the layers run in: [(layer index, pass number or None)], the pass number
+    given for the first layer of every pass of the looped run [start, stop)."""
+    n = len(layers)
+    if not loop:
+        return [(i, None) for i in range(n)]
+    a, b, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
+    if not (0 <= a < b <= n and times >= 1):
+        raise ValueError(f"bad loop {loop!r} over {n} layers")
+    runs = [(i, None) for i in range(a)]
+    for t in range(times):
+        runs += [(i, t if i == a else None) for i in range(a, b)]
+    return runs + [(i, None) for i in range(b, n)]
+
+
+def _mirorax_layer(e: dict) -> LayerSpec:
+    m = e["mixer"]
+    if e["type"] == "attention":
+        s = LayerSpec(MIX_ATTN, heads=m["heads"], kv_heads=m.get("kv_heads", m["heads"]), dim=m["dim"], vdim=m["vdim"],
+                      attn_scale=float(m["scale"]), mask_kind=MASK_CAUSAL, out_gate=GATE_ELEMENT, in_biased=True,
+                      o_biased=True)
+    elif e["type"] == "latent_attention":
+        rot = m["rot"]
+        s = LayerSpec(MIX_LATENT, heads=m["heads"], dim=m["dim"], vdim=m["vdim"], kv_rank=m["kv_rank"], q_rank=0,
+                      rot_dim=int(m["rot_dim"]), attn_scale=float(m["scale"]), mask_kind=MASK_WINDOW,
+                      mask_size=int(m["mask"]["size"]), rot_dims=int(rot["dims"]), rot_base=float(rot["base"]),
+                      sink=1, sink_learned=True)
+    else:
+        raise ValueError(f"unknown mixer type {e['type']!r}")
+    mlp = e.get("mlp")
+    if mlp:
+        if mlp["kind"] == "dense":
+            s.ff_kind, s.ff, s.limit, s.ff_act = FF_DENSE, mlp["ff"], float(mlp["limit"]), ACT_CLAMP
+        elif mlp["kind"] == "moe":
+            r = mlp["router"]
+            s.ff_kind, s.ff, s.ff_act = FF_MOE, mlp["expert"]["ff"], ACT_SILU
+            s.experts, s.top = r["experts"], r["top"]
+            s.router_kind, s.router_biased = ROUTER_TOP_SOFTMAX, True
+            if mlp.get("shared"):
+                s.shared_ff, s.shared_gated = mlp["shared"]["ff"], False
+        else:
+            raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+    return s
+
+
+def mirorax_config(cfg: dict, max_tokens: int = 4096, weight_dtype: int = M.BF16) -> LayeredConfig:
+    """config.json of a Mirorax checkpoint -> LayeredConfig whose layers are the layer RUNS (the
+    looped run unrolled; a repeated run shares the tensors of its first pass). Every size and
+    every constant that can differ between models of the design is read from cfg."""
+    first = {}
+    runs = []
+    for i, step in unroll_loop(cfg["layers"], cfg.get("loop")):
+        s = _mirorax_layer(cfg["layers"][i])
+        s.pre_added = step is not None
+        s.shares = first.get(i, -1)
+        first.setdefault(i, len(runs))
+        runs.append(s)
+    return LayeredConfig(
+        arch="Mirorax", width=cfg["width"], vocab=cfg["vocab"], layers=runs, embed_scale=1.0,
+        norm_eps=float(cfg["norm"]["eps"]), max_tokens=max_tokens, weight_dtype=weight_dtype, norm_kind=NORM_RMS,
+        pre_norm=True, pos_embed=False, block_kind=BLOCK_PARALLEL,
+    )
+
+
+def mirorax_tensor_shapes(cfg: dict) -> dict:
+    """Checkpoint tensor name -> shape for a Mirorax config.json."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W), "final.norm": (W,), "head": (cfg["vocab"], W)}
+    if cfg.get("loop"):
+        out["loop.step"] = (cfg["loop"]["times"], W)
+    for i, e in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", e["mixer"]
+        x = p + "mix."
+        out[p + "norm1"] = out[p + "ls1"] = (W,)
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        if e["type"] == "attention":
+            G = m.get("kv_heads", H)
+            for n, rows in (("q", H * D), ("k", G * D), ("v", G * V)):
+                out[x + n], out[x + n + ".b"] = (rows, W), (rows,)
+            out[x + "g"], out[x + "o"], out[x + "o.b"] = (H * V, W), (W, H * V), (W,)
+        else:
+            R, rank = m["rot_dim"], m["kv_rank"]
+            out[x + "q"], out[x + "dkv"], out[x + "dkv.norm"] = (H * (D + R), W), (rank + R, W), (rank,)
+            out[x + "uk"], out[x + "uv"], out[x + "sink"], out[x + "o"] = (H * D, rank), (H * V, rank), (H,), (W, H * V)
+        mlp = e.get("mlp")
+        if not mlp:
+            continue
+        out[p + "ls2"] = (W,)
+        f = p + "mlp."
+        if mlp["kind"] == "dense":
+            out[f + "gate"] = out[f + "up"] = (mlp["ff"], W)
+            out[f + "down"] = (W, mlp["ff"])
+        else:
+            ff, E = mlp["expert"]["ff"], mlp["router"]["experts"]
+            for k in range(E):
+                out[f"{f}e{k}.gate"] = out[f"{f}e{k}.up"] = (ff, W)
+                out[f"{f}e{k}.down"] = (W, ff)
+            out[f + "router"], out[f + "router.b"] = (E, W), (E,)
+            if mlp.get("shared"):
+                sf = mlp["shared"]["ff"]
+                out[f + "shared.gate"] = out[f + "shared.up"] = (sf, W)
+                out[f + "shared.down"] = (W, sf)
+    return out
+
+
+def mirorax_pack(c: LayeredConfig, t: dict, cfg: dict = None) -> dict:
+    """Checkpoint tensors -> the engine's tensors (see sinulorn_pack), one dict per layer run;
+    a repeated run holds the very arrays of its first pass (uploaded once) and its own pre_add."""
+    dt = c.weight_dtype
+    order = unroll_loop(cfg["layers"], cfg.get("loop"))
+
+    def w(*names):
+        parts = [_as_weight(t[n], dt) for n in names]
+        return parts[0] if len(parts) == 1 else np.ascontiguousarray(np.concatenate(parts, axis=0))
+
+    def f(name):
+        return np.ascontiguousarray(_as_f32(t[name]))
+
+    runs = []
+    for r, (l, (i, step)) in enumerate(zip(c.layers, order)):
+        own = {}
+        if step is not None:
+            own["pre_add"] = np.ascontiguousarray(f("loop.step")[step])
+        if l.shares >= 0:
+            d = {k: v for k, v in runs[l.shares].items() if k != "pre_add"}
+            d.update(own)
+            runs.append(d)
+            continue
+        p, x, m = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        d = dict(own, norm1=f(p + "norm1"), ls1=f(p + "ls1"))
+        if l.mixer == MIX_ATTN:
+            d["w_in"] = w(x + "q", x + "k", x + "v", x + "g")
+            b = np.zeros(l.in_rows, np.float32)  # the gate rows have no bias
+            qkv = np.concatenate([f(x + "q.b"), f(x + "k.b"), f(x + "v.b")])
+            b[:qkv.size] = qkv
+            d.update(in_bias=b, o_bias=f(x + "o.b"))
+        else:
+            d["w_in"] = w(x + "q", x + "dkv")
+            d.update(kv_norm=f(x + "dkv.norm"), sink_w=f(x + "sink"), w_uv=w(x + "uv"))
+            uk = _as_weight(t[x + "uk"], dt).reshape(l.heads, l.dim, l.kv_rank)
+            d["w_ukt"] = np.ascontiguousarray(uk.transpose(0, 2, 1))
+        d["w_o"] = w(x + "o")
+        if l.ff_kind != FF_NONE:
+            d["ls2"] = f(p + "ls2")
+        if l.ff_kind == FF_DENSE:
+            d.update(w_gate=w(m + "gate"), w_up=w(m + "up"), w_down=w(m + "down"))
+        elif l.ff_kind == FF_MOE:
+            d.update(router=f(m + "router"), router_bias=f(m + "router.b"))
+            for k in ("gate", "up", "down"):
+                d["w_" + k] = np.ascontiguousarray(
+                    np.stack([_as_weight(t[f"{m}e{e}.{k}"], dt) for e in range(l.experts)]))
+            if l.shared_ff:
+                d.update(ws_gate=w(m + "shared.gate"), ws_up=w(m + "shared.up"), ws_down=w(m + "shared.down"))
+        want = packed_shapes(c, l)
+        if set(want) != set(d):
+            raise ValueError(f"layer {i}: packed tensors {sorted(d)} do not match the configuration's {sorted(want)}")
+        for k, (shape, _) in want.items():
+            if tuple(d[k].shape) != tuple(shape):
+                raise ValueError(f"layer {i}: tensor {k} has shape {d[k].shape}, the configuration gives {shape}")
+        runs.append(d)
+    return {"embed": w("embed"), "final_norm": f("final.norm"), "head": w("head"), "layers": runs}
+
+
+def mirorax_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0) -> dict:
+    """Random checkpoint tensors for a Mirorax config.json, as float32 arrays already rounded
+    to bf16 values (the f32 and bf16 engines and a float64 restatement see the same weights)."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in mirorax_tensor_shapes(cfg).items():
+        leaf = name.split(".")[-1]
+        if leaf == "norm1" or name.endswith(".norm"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif leaf in ("ls1", "ls2"):
+            a = rng.uniform(0.3, 1.1, shape) * rng.choice([-1.0, 1.0], shape)
+        elif leaf == "b":
+            a = 0.3 * rng.standard_normal(shape)
+        elif leaf == "sink":
+            a = rng.uniform(-1.0, 2.0, shape)
+        elif leaf == "step":
+            a = 0.3 * rng.standard_normal(shape)
+        elif leaf == "embed":
+            a = 0.5 * rng.standard_normal(shape)
+        else:
+            a = gain * rng.standard_normal(shape) / np.sqrt(shape[-1])
+        out[name] = bf16_to_f32(f32_to_bf16(a.astype(np.float32))).reshape(shape)
+    return out
+
+
 # ------------------------------------------------------------------ registry
 # design name (config.json "architecture") -> (config reader, weight packer)
-DESIGNS = {"Sinulorn": (sinulorn_config, sinulorn_pack), "Lenuzen": (lenuzen_config, lenuzen_pack)}
+DESIGNS = {"Sinulorn": (sinulorn_config, sinulorn_pack), "Lenuzen": (lenuzen_config, lenuzen_pack),
+           "Mirorax": (mirorax_config, lambda c, t, cfg=None: mirorax_pack(c, t, cfg))}
 
 
 def read_checkpoint(path: str, max_tokens: int = 4096, weight_dtype: int = M.BF16):
@@ -522,6 +769,6 @@ def read_checkpoint(path: str, max_tokens: int = 4096, weight_dtype: int = M.BF1
     yd = read_yalm(os.path.join(path, "model.safetensors"))
     try:
         t = {k: np.asarray(v.data).reshape(v.shape) for k, v in yd.tensors.items()}
-        return c, packer(c, t)
+        return c, (packer(c, t, cfg) if arch == "Mirorax" else packer(c, t))
     finally:
         yd.close()

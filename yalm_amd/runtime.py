@@ -141,15 +141,17 @@ _sig("yalm_attn_wo_plan", c_int, [c_void_p, c_int, ctypes.POINTER(c_int), ctypes
 class SeqLayer(ctypes.Structure):
     """yalm_seq_layer."""
 
-    INTS = ("mixer", "heads", "kv_heads", "dim", "vdim", "kv_rank", "q_rank", "kv_from")
-    PTRS = ("norm1", "norm1b", "norm2", "norm2b", "q_norm", "kv_norm", "in_bias", "head_temp", "talk", "conv_w", "conv_b", "gate_a",
+    INTS = ("mixer", "heads", "kv_heads", "dim", "vdim", "kv_rank", "q_rank", "kv_from", "rot_dim")
+    PTRS = ("norm1", "norm1b", "norm2", "norm2b", "ls1", "ls2", "pre_add", "sink_w", "o_bias", "router_bias",
+            "q_norm", "kv_norm", "in_bias", "head_temp", "talk", "conv_w", "conv_b", "gate_a",
             "gate_a_b", "gate_i", "gate_i_b", "lam", "a_log", "dt_bias", "out_norm", "router", "shared_sg",
             "w_in", "w_uq", "w_ukt", "w_uv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
     _fields_ = (
         [(n, c_int) for n in INTS] + [("attn_scale", c_float), ("rec_width", c_int), ("blocks", c_int), ("conv", c_int),
                                       ("ff_kind", c_int), ("ff", c_int), ("experts", c_int), ("top", c_int),
                                       ("groups", c_int), ("groups_keep", c_int), ("router_scale", c_float),
-                                      ("limit", c_float), ("shared_ff", c_int), ("shared_limit", c_float)]
+                                      ("limit", c_float), ("shared_ff", c_int), ("shared_limit", c_float),
+                                      ("ff_act", c_int), ("router_kind", c_int)]
         + [(n, c_int) for n in ("mask_kind", "mask_size", "qk_norm", "v_norm", "sink", "out_gate", "rot_dims",
                                 "rot_orig")]
         + [(n, c_float) for n in ("rot_base", "rot_factor", "rot_fast", "rot_slow")]
@@ -160,7 +162,7 @@ class SeqLayer(ctypes.Structure):
 class SeqConfig(ctypes.Structure):
     _fields_ = [("width", c_int), ("vocab", c_int), ("n_layers", c_int), ("max_tokens", c_int),
                 ("embed_scale", c_float), ("norm_eps", c_float), ("weight_dtype", c_int), ("norm_kind", c_int),
-                ("pre_norm", c_int), ("pos_embed", c_int), ("logit_scale", c_float)]
+                ("pre_norm", c_int), ("pos_embed", c_int), ("logit_scale", c_float), ("block_kind", c_int)]
 
 
 class SeqWeights(ctypes.Structure):
@@ -659,8 +661,14 @@ class SeqModel:
         for k in ("embed", "final_norm", "head"):
             # a tied head aliases the embedding table instead of a second upload
             self.ptrs[k] = self.ptrs["embed"] if k == "head" and packed[k] is packed["embed"] else self._up(packed[k])
+        seen = {}  # layer runs that share tensors hold the same arrays: one upload each
         for d in packed["layers"]:
-            self.layer_ptrs.append({k: self._up(a) for k, a in d.items()})
+            ptrs = {}
+            for k, a in d.items():
+                if id(a) not in seen:
+                    seen[id(a)] = self._up(a)
+                ptrs[k] = seen[id(a)]
+            self.layer_ptrs.append(ptrs)
         return self
 
     @classmethod
@@ -692,6 +700,8 @@ class SeqModel:
                 scale, off = 1.7 / np.sqrt(fan_in or shape[-1]), 0.0
             elif leaf.startswith("norm") or leaf in ("q_norm", "kv_norm", "out_norm", "final_norm", "head_temp"):
                 scale, off = 0.2, 1.0
+            elif leaf in ("ls1", "ls2"):
+                scale, off = 0.2, 0.6
             elif leaf == "conv_w":
                 scale, off = 0.5, 0.0
             elif leaf in ("lam", "a_log", "dt_bias"):
@@ -705,8 +715,10 @@ class SeqModel:
         self.ptrs["final_norm"] = make("final_norm", (cfg.width,), "f")
         self.ptrs["head"] = self.ptrs["embed"] if cfg.tied_head else make("head", (cfg.vocab, cfg.width), "w")
         for i, l in enumerate(cfg.layers):
-            self.layer_ptrs.append({k: make(f"l{i}.{k}", shape, kind)
-                                    for k, (shape, kind) in layered.packed_shapes(cfg, l).items()})
+            ptrs = {k: make(f"l{i}.{k}", shape, kind) for k, (shape, kind) in layered.packed_shapes(cfg, l).items()}
+            if l.shares >= 0:  # a repeated run: the first pass's tensors, its own pre_add
+                ptrs = {**{k: v for k, v in self.layer_ptrs[l.shares].items() if k != "pre_add"}, **ptrs}
+            self.layer_ptrs.append(ptrs)
         check(lib.yalm_stream_sync(None))
         return self
 
@@ -720,7 +732,8 @@ class SeqModel:
                 else:
                     setattr(arr[i], name, getattr(l, name))
         sc = SeqConfig(cfg.width, cfg.vocab, len(cfg.layers), cfg.max_tokens, cfg.embed_scale, cfg.norm_eps,
-                       cfg.weight_dtype, cfg.norm_kind, int(cfg.pre_norm), int(cfg.pos_embed), cfg.logit_scale)
+                       cfg.weight_dtype, cfg.norm_kind, int(cfg.pre_norm), int(cfg.pos_embed), cfg.logit_scale,
+                       cfg.block_kind)
         sw = SeqWeights(self.ptrs["embed"], self.ptrs["final_norm"], self.ptrs["head"], arr)
         return sc, sw, arr
 
