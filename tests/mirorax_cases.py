@@ -79,3 +79,9 @@ DENSE_ONLY = config([
 
 ALL = {"only_attn": ONLY_ATTN, "only_latent": ONLY_LATENT, "only_dense": ONLY_DENSE, "only_moe": ONLY_MOE,
        "only_loop": ONLY_LOOP, "loop_once": LOOP_ONCE, "mixed": MIXED, "odd": ODD, "wide": WIDE, "dense_only": DENSE_ONLY}
+
+
+def tokens(cfg, n, seed=0):
+    import numpy as np
+
+    return np.random.default_rng(2000 + seed).integers(0, cfg["vocab"], n).tolist()

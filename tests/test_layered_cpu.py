@@ -170,6 +170,124 @@ def test_lenuzen_restatement_is_causal_and_masks_hold():
     assert np.allclose(p, [[1 / 3, 1 / 3, 0.0]])
 
 
+# ------------------------------------------------------------------ Mirorax
+def test_mirorax_config_reads_every_size_and_constant():
+    import mirorax_cases as MC
+
+    c = Ly.mirorax_config(MC.MIXED, max_tokens=300)
+    assert (c.arch, c.width, c.vocab, c.embed_scale, c.norm_eps, c.max_tokens, c.logit_scale) == (
+        "Mirorax", 96, 211, 1.0, 1e-5, 300, 1.0)
+    assert (c.norm_kind, c.pre_norm, c.pos_embed, c.tied_head, c.block_kind) == (
+        Ly.NORM_RMS, True, False, False, Ly.BLOCK_PARALLEL)
+    # layers 1..3 are walked twice: 6 layers, 9 runs; the repeated runs share their first pass
+    assert [l.shares for l in c.layers] == [-1, -1, -1, -1, 1, 2, 3, -1, -1]
+    assert [l.pre_added for l in c.layers] == [False, True, False, False, True, False, False, False, False]
+    a0, l1, a2, l3 = c.layers[:4]
+    assert (a0.mixer, a0.heads, a0.kv_heads, a0.dim, a0.vdim, a0.attn_scale, a0.mask_kind, a0.out_gate, a0.sink) == (
+        Ly.MIX_ATTN, 4, 2, 24, 40, 0.21, Ly.MASK_CAUSAL, Ly.GATE_ELEMENT, 0)
+    assert (a0.in_biased, a0.o_biased, a0.rot_dims, a0.ff_kind, a0.ff, a0.limit, a0.ff_act) == (
+        True, True, 0, Ly.FF_DENSE, 72, 1.25, Ly.ACT_CLAMP)
+    assert a0.in_rows == 4 * 24 + 2 * (24 + 40) + 4 * 40
+    assert (l1.mixer, l1.heads, l1.dim, l1.rot_dim, l1.vdim, l1.kv_rank, l1.q_rank, l1.mask_kind, l1.mask_size) == (
+        Ly.MIX_LATENT, 3, 24, 8, 40, 32, 0, Ly.MASK_WINDOW, 9)
+    assert (l1.sink, l1.sink_learned, l1.rot_dims, l1.rot_base, l1.attn_scale) == (1, True, 8, 10000.0, 0.19)
+    assert l1.in_rows == 3 * (24 + 8) + 32 + 8 and l1.mix_out == 3 * 40
+    assert (l1.ff_kind, l1.ff, l1.experts, l1.top, l1.shared_ff, l1.shared_gated, l1.ff_act, l1.router_kind,
+            l1.router_biased) == (Ly.FF_MOE, 40, 6, 2, 24, False, Ly.ACT_SILU, Ly.ROUTER_TOP_SOFTMAX, True)
+    assert (a2.top, a2.shared_ff, a2.kv_heads) == (1, 0, 6)
+    assert (l3.rot_dim, l3.rot_dims, l3.rot_base, l3.mask_size, l3.ff_kind) == (16, 8, 500.0, 1, Ly.FF_NONE)
+    assert c.layers[7].limit == 0.75 and c.layers[8].top == 5
+
+
+def test_mirorax_loops_unroll():
+    assert Ly.unroll_loop([0] * 3, None) == [(0, None), (1, None), (2, None)]
+    assert Ly.unroll_loop([0] * 3, {"start": 0, "stop": 3, "times": 1}) == [(0, 0), (1, None), (2, None)]
+    assert Ly.unroll_loop([0] * 4, {"start": 1, "stop": 3, "times": 3}) == [
+        (0, None), (1, 0), (2, None), (1, 1), (2, None), (1, 2), (2, None), (3, None)]
+    assert Ly.unroll_loop([0] * 2, {"start": 1, "stop": 2, "times": 2}) == [(0, None), (1, 0), (1, 1)]
+    with pytest.raises(ValueError):
+        Ly.unroll_loop([0] * 2, {"start": 1, "stop": 3, "times": 2})
+    import mirorax_cases as MC
+    import mirorax_ref as MR
+
+    for cfg in MC.ALL.values():
+        assert MR.layer_runs(cfg) == Ly.unroll_loop(cfg["layers"], cfg.get("loop"))
+
+
+def test_mirorax_unknown_names_are_refused():
+    import mirorax_cases as MC
+
+    with pytest.raises(ValueError):
+        Ly.mirorax_config(MC.config([("attention_2", MC.attn(), None)]))
+    with pytest.raises(ValueError):
+        Ly.mirorax_config(MC.config([("attention", MC.attn(), {"kind": "plain", "ff": 8})]))
+
+
+def test_mirorax_pack_concatenates_and_shares_repeated_runs():
+    import mirorax_cases as MC
+
+    cfg = MC.MIXED
+    t = Ly.mirorax_random_tensors(cfg, seed=3)
+    assert set(t) == set(Ly.mirorax_tensor_shapes(cfg))
+    for wdt in (M.F32, M.BF16):
+        c = Ly.mirorax_config(cfg, weight_dtype=wdt)
+        p = Ly.mirorax_pack(c, t, cfg)
+        f = (lambda a: a) if wdt == M.F32 else Ly.bf16_to_f32
+        assert len(p["layers"]) == 9 and p["head"] is not p["embed"]
+        d0, l0 = p["layers"][0], c.layers[0]
+        assert np.array_equal(f(d0["w_in"]), np.concatenate([t["l0.mix." + n] for n in ("q", "k", "v", "g")]))
+        nb = l0.in_rows - l0.heads * l0.vdim
+        assert np.array_equal(d0["in_bias"][:nb], np.concatenate([t["l0.mix." + n + ".b"] for n in ("q", "k", "v")]))
+        assert not d0["in_bias"][nb:].any() and np.array_equal(d0["o_bias"], t["l0.mix.o.b"])
+        assert np.array_equal(d0["ls1"], t["l0.ls1"]) and np.array_equal(d0["ls2"], t["l0.ls2"]) and "pre_add" not in d0
+        d1, l1 = p["layers"][1], c.layers[1]
+        assert np.array_equal(f(d1["w_in"]), np.concatenate([t["l1.mix.q"], t["l1.mix.dkv"]]))
+        uk = t["l1.mix.uk"].reshape(l1.heads, l1.dim, l1.kv_rank)
+        assert np.array_equal(f(d1["w_ukt"]), uk.transpose(0, 2, 1))
+        assert np.array_equal(d1["sink_w"], t["l1.mix.sink"]) and np.array_equal(d1["router_bias"], t["l1.mlp.router.b"])
+        assert np.array_equal(f(d1["w_gate"][4]), t["l1.mlp.e4.gate"]) and "shared_sg" not in d1
+        # the loop: pass t of layers 1..3 adds step[t] before layer 1; later passes hold the first pass's arrays
+        assert np.array_equal(d1["pre_add"], t["loop.step"][0]) and np.array_equal(p["layers"][4]["pre_add"], t["loop.step"][1])
+        for r, first in ((4, 1), (5, 2), (6, 3)):
+            for k, a in p["layers"][r].items():
+                assert k == "pre_add" or a is p["layers"][first][k]
+        assert "pre_add" not in p["layers"][5] and "ls2" not in p["layers"][3]
+        for l, d in zip(c.layers, p["layers"]):
+            own = set(Ly.packed_shapes(c, l))
+            assert own <= set(d) and (l.shares >= 0 or own == set(d))
+
+
+def test_mirorax_restatement_is_causal_and_its_window_and_sink_hold():
+    """The restatement itself: logits at t do not depend on later tokens; a one-layer latent
+    model's logits at t do not depend on tokens its window has left behind; the sink takes
+    its share of the softmax."""
+    import mirorax_cases as MC
+    import mirorax_ref as MR
+
+    cfg = MC.MIXED
+    w = {k: v.astype(np.float64) for k, v in Ly.mirorax_random_tensors(cfg, seed=4).items()}
+    a = MC.tokens(cfg, 40, 1)
+    b = list(a)
+    b[30] = (b[30] + 1) % cfg["vocab"]
+    ra, rb = MR.forward(cfg, w, a), MR.forward(cfg, w, b)
+    assert np.array_equal(ra[:30], rb[:30]) and not np.allclose(ra[30], rb[30])
+    one = MC.ONLY_LATENT
+    size = one["layers"][0]["mixer"]["mask"]["size"]
+    w1 = {k: v.astype(np.float64) for k, v in Ly.mirorax_random_tensors(one, seed=5).items()}
+    a = MC.tokens(one, 30, 2)
+    b = list(a)
+    b[10] = (b[10] + 1) % one["vocab"]
+    ra, rb = MR.forward(one, w1, a), MR.forward(one, w1, b)
+    assert not np.allclose(ra[10 + size - 1], rb[10 + size - 1]) and np.allclose(ra[10 + size:], rb[10 + size:], atol=1e-12)
+    m = MR.visible(3, 6)
+    assert m[5, 3] and not m[5, 2] and m[2, 0] and not m[2, 3]
+    p = MR.softmax_rows(np.zeros((1, 1, 3)), np.array([[[True, True, False]]]), sink=np.array([np.log(2.0)]))
+    assert np.allclose(p, [[[0.25, 0.25, 0.0]]])
+    idx, wt = MR.route({"r.router": np.eye(4), "r.router.b": np.array([0.0, 0.0, 5.0, 0.0])}, "r.",
+                       np.array([[3.0, 1.0, 0.0, 2.0]]), 2)
+    assert idx.tolist() == [[2, 0]] and np.allclose(wt, [[np.exp(2) / (1 + np.exp(2)), 1 / (1 + np.exp(2))]])
+
+
 def test_bench_stacks_are_valid_layer_list_configurations():
     """The stacks bench.py --layered times: every layer's packed tensor set is well formed at
     every benchmarked width, and mixed-score layers keep their key row within the MFMA
