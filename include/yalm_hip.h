@@ -413,7 +413,10 @@ typedef struct yalm_seq_layer {
 	                      attn: [heads dim + kv_heads dim + kv_heads vdim (+ heads | heads vdim if out_gate)][width] (q, k, v, gate) */
 	const void *w_uq;  /* latent: [heads dim][q_rank] (unused with q_rank = 0) */
 	const void *w_ukt; /* latent: [heads][kv_rank][dim], the key up-projection transposed per head */
-	const void *w_uv;  /* latent: [heads vdim][kv_rank] */
+	const void *w_uv;  /* latent: [heads vdim][kv_rank]; NULL with w_ukv: its last heads vdim rows */
+	const void *w_ukv; /* latent with q_rank = 0, or NULL: [heads dim + heads vdim][kv_rank], the key and the value
+	                      up-projections stacked; portions then expand the cached latents they see into per-head keys
+	                      and values instead of attending over the latents */
 	const void *w_o;   /* [width][heads vdim | rec_width] */
 	const void *w_gate, *w_up, *w_down; /* dense: [ff][width] x2, [width][ff]; moe: the same per expert, stacked;
 	                                       plain: w_down gelu(w_up x), no w_gate */

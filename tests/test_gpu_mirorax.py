@@ -484,7 +484,7 @@ def test_new_options_combine_freely(rt, dtype):
     as_w = (lambda a: np.ascontiguousarray(a, np.float32)) if dtype == "f32" else Ly.f32_to_bf16
     l0 = {"norm1": t["norm1.0"], "norm1b": t["norm1b.0"], "norm2": t["norm2.0"], "norm2b": t["norm2b.0"],
           "w_in": as_w(np.concatenate([t["q0"], t["dkv0"]])), "kv_norm": t["kvn0"],
-          "w_ukt": as_w(np.ascontiguousarray(t["uk0"].reshape(H, D, rank).transpose(0, 2, 1))), "w_uv": as_w(t["uv0"]),
+          "w_ukt": as_w(np.ascontiguousarray(t["uk0"].reshape(H, D, rank).transpose(0, 2, 1))), "w_ukv": as_w(np.concatenate([t["uk0"], t["uv0"]])),
           "w_o": as_w(t["o0"]), "w_gate": as_w(t["gate0"]), "w_up": as_w(t["up0"]), "w_down": as_w(t["down0"])}
     l1 = {"norm1": t["norm1.1"], "norm1b": t["norm1b.1"], "w_in": as_w(np.concatenate([t["q1"], t["k1"], t["v1"], t["g1"]])),
           "w_o": as_w(t["o1"]), "o_bias": t["ob1"]}
@@ -550,17 +550,25 @@ def test_prompt_longer_than_one_internal_portion(rt, dtype):
         model.close()
 
 
-def test_large_latent_sizes(rt):
-    """A latent of 256 + 64 rotated entries and 16 heads: key rows of more than 256 entries,
-    portions on the matrix cores (bf16) and on the f32 tiles, single tokens through key splits."""
-    cfg = C.config([(C.L, C.latent(heads=16, dim=32, rot_dim=64, vdim=32, kv_rank=256, size=200, scale=0.08, rot_dims=64),
-                     C.dense(ff=64))], width=128, vocab=101)
+LARGE = {
+    # key rows of more than 256 entries: long portions expand the latents into per-head keys and
+    # values, short ones and single tokens attend over the latent rows (f32 tiles, key splits)
+    "rank256": C.latent(heads=16, dim=32, rot_dim=64, vdim=32, kv_rank=256, size=200, scale=0.08, rot_dims=64),
+    # latent rows too long for the f32 tiles: every portion of two tokens or more expands; single
+    # tokens take blocks of 16 of the 24 heads per workgroup
+    "rank512": C.latent(heads=24, dim=16, rot_dim=64, vdim=24, kv_rank=512, size=150, scale=0.06, rot_dims=32),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LARGE))
+def test_large_latent_sizes(rt, name):
+    cfg = C.config([(C.L, LARGE[name], C.dense(ff=64))], width=128, vocab=101)
     for dtype in ("f32", "bf16"):
         model, dec, w = build(rt, cfg, wdt_of(dtype), seed=22, max_tokens=400)
         try:
             tok = C.tokens(cfg, 330, 22)
             ref = R.forward(cfg, w, tok)
-            assert agrees(run_portions(dec, tok, [300, 5] + [1] * 25), ref, dtype, cfg)
+            assert agrees(run_portions(dec, tok, [270, 5, 2, 20, 9] + [1] * 24), ref, dtype, cfg)
         finally:
             dec.close()
             model.close()

@@ -244,6 +244,7 @@ def test_mirorax_pack_concatenates_and_shares_repeated_runs():
         assert np.array_equal(f(d1["w_in"]), np.concatenate([t["l1.mix.q"], t["l1.mix.dkv"]]))
         uk = t["l1.mix.uk"].reshape(l1.heads, l1.dim, l1.kv_rank)
         assert np.array_equal(f(d1["w_ukt"]), uk.transpose(0, 2, 1))
+        assert np.array_equal(f(d1["w_ukv"]), np.concatenate([t["l1.mix.uk"], t["l1.mix.uv"]])) and "w_uv" not in d1
         assert np.array_equal(d1["sink_w"], t["l1.mix.sink"]) and np.array_equal(d1["router_bias"], t["l1.mlp.router.b"])
         assert np.array_equal(f(d1["w_gate"][4]), t["l1.mlp.e4.gate"]) and "shared_sg" not in d1
         # the loop: pass t of layers 1..3 adds step[t] before layer 1; later passes hold the first pass's arrays

@@ -53,6 +53,12 @@ struct yalm_seq_s {
 	float *logits = nullptr;     // [LOGIT_ROWS][vocab]
 	int *idx = nullptr, *counts = nullptr, *lists = nullptr;
 	float *wt = nullptr, *sgate = nullptr;
+	int cur_pos = 0;             // the position the portion being enqueued starts at (host copy of st->pos)
+	// latent attention with directly projected queries, portions: the visible positions' latents
+	// as f32, their expanded keys | values as f32, then per-head key and value rows in the cache's type
+	float *ex_c = nullptr, *ex_kv = nullptr;
+	void *ex_k = nullptr, *ex_v = nullptr;
+	int ex_rows = 0;
 	float *att_part = nullptr;   // latent attention: per (row, key split) partial sums, maximum, sum
 	int att_splits = 1;          // key splits of single-token / short-portion attention
 	float *arena = nullptr;      // every recurrent and convolution state of the sequence
@@ -138,7 +144,7 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 				set_err(at + "heads x kv_rank above 16384 is not implemented by the attention kernels");
 				return YALM_ERR_UNSUPPORTED;
 			}
-			ARGCHK(l.kv_norm && l.w_ukt && l.w_uv, at + "missing latent attention tensors");
+			ARGCHK(l.kv_norm && l.w_ukt && (l.w_uv || l.w_ukv), at + "missing latent attention tensors");
 			ARGCHK(l.mask_kind == YALM_MASK_CAUSAL || ((l.mask_kind == YALM_MASK_WINDOW || l.mask_kind == YALM_MASK_CHUNK) && l.mask_size > 0),
 			       at + "bad attention mask");
 			ARGCHK(l.rot_dims >= 0 && l.rot_dims <= l.rot_dim && l.rot_dims % 2 == 0 && (l.rot_dims == 0 || l.rot_base > 0.0f),
@@ -311,7 +317,8 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	for (const yalm_seq_layer &l : q->L) {
 		zw = std::max(zw, in_rows(l));
 		if (l.mixer == YALM_MIX_LATENT) {
-			bw = std::max({bw, (size_t)l.heads * l.dim, (size_t)l.heads * (l.kv_rank + l.rot_dim), (size_t)l.heads * l.vdim, (size_t)l.q_rank});
+			bw = std::max({bw, (size_t)l.heads * (l.dim + l.rot_dim), (size_t)l.heads * (l.kv_rank + l.rot_dim),
+			               (size_t)l.heads * l.vdim, (size_t)l.q_rank});
 		} else if (l.mixer == YALM_MIX_RGLRU) {
 			bw = std::max(bw, (size_t)l.rec_width);
 			arena += (size_t)l.rec_width + (size_t)(l.conv - 1) * l.rec_width;
@@ -370,7 +377,7 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 				continue;
 			const int span = l.mask_kind == YALM_MASK_CAUSAL ? c.max_tokens : std::min(c.max_tokens, l.mask_size + GEMV_MAX_M);
 			q->attn_splits[i] = std::max(1, std::min(64, cdiv(span, SA_KT)));
-			const int vd = l.mixer == YALM_MIX_ATTN ? l.vdim : l.kv_rank; // the attention's value size
+			const int vd = l.mixer == YALM_MIX_ATTN ? l.vdim : std::max(l.kv_rank, l.vdim); // the attention's value size
 			part = std::max(part, (size_t)GEMV_MAX_M * l.heads * q->attn_splits[i] * (att_rank4(vd) + 4));
 		}
 		STRY(sallocT(q, &q->att_part, part));
@@ -427,6 +434,26 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 			off += (size_t)l.heads * l.dim * l.vdim;
 			q->conv[i] = q->arena + off;
 			off += (size_t)(l.conv - 1) * cc;
+		}
+	}
+	{ // expansion buffers: the most positions a portion's rows see, over the layers that expand
+		size_t rows = 0, nc = 0, nkv = 0, nk = 0, nv = 0;
+		for (const yalm_seq_layer &l : q->L)
+			if (latent_direct(l) && l.w_ukv) {
+				const size_t span = l.mask_kind == YALM_MASK_CAUSAL ? (size_t)c.max_tokens : (size_t)l.mask_size + q->cap;
+				rows = std::max(rows, std::min((size_t)c.max_tokens, span));
+				nc = std::max(nc, (size_t)l.kv_rank);
+				nkv = std::max(nkv, (size_t)l.heads * (l.dim + l.vdim));
+				nk = std::max(nk, (size_t)l.heads * (l.dim + l.rot_dim));
+				nv = std::max(nv, (size_t)l.heads * l.vdim);
+			}
+		if (rows) {
+			q->ex_rows = (int)rows;
+			if (bf)
+				STRY(sallocT(q, &q->ex_c, rows * nc));
+			STRY(sallocT(q, &q->ex_kv, rows * nkv));
+			STRY(salloc(q, &q->ex_k, rows * nk * (bf ? 2 : 4)));
+			STRY(salloc(q, &q->ex_v, rows * nv * (bf ? 2 : 4)));
 		}
 	}
 	for (int i = 0; i < c.n_layers; ++i)
@@ -740,10 +767,11 @@ static int gemm_in(Seq *q, GemmArgs a) {
 }
 
 template <int KS>
-static int attn_mfma_launch(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
+static int attn_mfma_launch(Seq *q, const void *kc, const void *vc, int n, const AttnArgs &a, const float *Q,
+                            const float *gate, float *ctx) {
 	const int rep = a.H / a.G, HW = rep >= 4 ? 4 : (rep >= 2 ? 2 : 1), NT = cdiv(a.V, 16);
 	const dim3 g(cdiv(n, 16 * (4 / HW)), a.G, cdiv(rep, HW));
-	const uint16_t *Kc = (const uint16_t *)q->cache[li], *Vc = (const uint16_t *)q->vcache[li];
+	const uint16_t *Kc = (const uint16_t *)kc, *Vc = (const uint16_t *)vc;
 #define SAM_LAUNCH(N)                                                                                                  \
 	seq_attn_mfma_kernel<KS, N><<<g, SEQ_THREADS, 0, q->stream>>>(Q, Kc, Vc, a, n, HW, q->st, gate, ctx)
 	if (NT <= 2) SAM_LAUNCH(2);
@@ -754,27 +782,36 @@ static int attn_mfma_launch(Seq *q, int li, int n, const AttnArgs &a, const floa
 	return YALM_OK;
 }
 
+// kc / vc: the key and value rows, row = position (the layer's caches, or a portion's expanded
+// keys and values whose pointer is moved back by the first row's position)
 template <class CT>
-static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
+static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx,
+                       const void *kc = nullptr, const void *vc = nullptr) {
+	if (!kc) {
+		kc = q->cache[li];
+		vc = q->vcache[li];
+	}
 	const bool talk = a.talk != nullptr;
 	const int DK = talk ? a.G * a.D : a.D;
 	if (sizeof(CT) == 2 && n > GEMV_MAX_M && DK <= 512 && a.V <= 128) { // portions over bf16 caches: the MFMA form
 		const int ks = cdiv(DK, 32);
-		if (ks <= 1) return attn_mfma_launch<1>(q, li, n, a, Q, gate, ctx);
-		if (ks <= 2) return attn_mfma_launch<2>(q, li, n, a, Q, gate, ctx);
-		if (ks <= 4) return attn_mfma_launch<4>(q, li, n, a, Q, gate, ctx);
-		if (ks <= 8) return attn_mfma_launch<8>(q, li, n, a, Q, gate, ctx);
-		return attn_mfma_launch<16>(q, li, n, a, Q, gate, ctx);
+		if (ks <= 1) return attn_mfma_launch<1>(q, kc, vc, n, a, Q, gate, ctx);
+		if (ks <= 2) return attn_mfma_launch<2>(q, kc, vc, n, a, Q, gate, ctx);
+		if (ks <= 4) return attn_mfma_launch<4>(q, kc, vc, n, a, Q, gate, ctx);
+		if (ks <= 8) return attn_mfma_launch<8>(q, kc, vc, n, a, Q, gate, ctx);
+		return attn_mfma_launch<16>(q, kc, vc, n, a, Q, gate, ctx);
 	}
 	const int Hb = a.H / a.G, Gb = talk ? a.G : 1, V4n = (a.V + 3) / 4, D4 = (a.D + 3) & ~3;
-	const CT *Kc = (const CT *)q->cache[li], *Vc = (const CT *)q->vcache[li];
+	const CT *Kc = (const CT *)kc, *Vc = (const CT *)vc;
 	const int rep = a.H / a.G;
-	const size_t dec_lds = sa_decode_lds_bytes(rep, DK, talk ? a.H * a.D : 0, a.H);
+	// many heads over one key/value head: blocks of SA_DEC_HB heads per workgroup
+	const int hz = !talk && rep > SA_DEC_HB ? cdiv(rep, SA_DEC_HB) : 1, hb = hz > 1 ? SA_DEC_HB : rep;
+	const size_t dec_lds = sa_decode_lds_bytes(hb, DK, talk ? a.H * a.D : 0, a.H);
 	if (n == 1 && !a.q_mixed && dec_lds <= 96 * 1024) { // a decoded token: lanes read the cache rows themselves
 		const int S = q->attn_splits[li];
-		const dim3 g(S, a.G);
+		const dim3 g(S, a.G, hz);
 		const size_t lds = dec_lds;
-		const int na = cdiv(rep * V4n, SEQ_THREADS);
+		const int na = cdiv(hb * V4n, SEQ_THREADS);
 #define SD_LAUNCH(NA)                                                                                                  \
 	do {                                                                                                               \
 		static bool attr_set = false;                                                                                  \
@@ -906,37 +943,43 @@ static int mixer_attn(Seq *q, int li, int n) {
 // the cache rows [c_j | k_rot_j] themselves and sums their first kv_rank entries: the softmax-
 // attention kernels with one key/value head, key size kv_rank + rot_dim, value size kv_rank,
 // the value rows aliasing the key rows.
+// Do the f32 FMA attention tiles fit in LDS for n tokens of H heads over G key/value heads?
+static bool attn_fma_fits(int H, int G, int D, int V, int n) {
+	const int Hb = H / G, D4 = (D + 3) & ~3;
+	int TQ = std::max(1, std::min(32 / std::max(Hb, 1), n));
+	while (TQ > 1 && (size_t)TQ * Hb * D4 * sizeof(float) > 64 * 1024)
+		--TQ;
+	return sa_lds_bytes(TQ * Hb, 1, D, V) <= 160 * 1024 - 64;
+}
+
 static int mixer_latent_direct(Seq *q, int li, int n) {
 	const yalm_seq_layer &l = q->L[li];
 	const yalm_seq_config &c = q->c;
 	const bool bf = c.weight_dtype == YALM_BF16;
 	const int zin = in_rows(l), H = l.heads, D = l.dim, R = l.rot_dim, V = l.vdim, rk = l.kv_rank, KR = rk + R;
 	float *qp = q->B[0], *qa = q->B[1], *ctx = q->B[2], *oh = q->B[3];
+	const void *w_uv = l.w_uv ? l.w_uv : (const char *)l.w_ukv + (size_t)H * D * rk * (bf ? 2 : 4);
+	// Portions expand the latents they see into per-head keys and values (one product with the
+	// stacked up-projections) and attend with ordinary heads of dim + rot_dim / vdim entries:
+	// fewer multiply-adds per (query, key) pair than over the latent (2 kv_rank + rot_dim), and
+	// head sizes the matrix-core attention takes. Single tokens and short portions attend over
+	// the latent itself, unless its rows are too long for the f32 tiles.
+	const int klo = attn_first_key(l.mask_kind, l.mask_size, q->cur_pos), rows = q->cur_pos + n - klo;
+	const bool absorbed_ok = n == 1 || (bf && n > GEMV_MAX_M && KR <= 512 && rk <= 128) || attn_fma_fits(H, 1, KR, rk, n);
+	const bool expand = l.w_ukv && n > 1 && rows <= q->ex_rows && (n >= 32 || !absorbed_ok);
 	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
 	const size_t rot_lds = (size_t)std::max(l.rot_dims, 2) * sizeof(float);
 	if (bf)
 		seq_latent_prep_kernel<uint16_t><<<n, SEQ_THREADS, rot_lds, q->stream>>>(
 		    q->Z, zin, H, D, R, rk, l.rot_dims, q->rot_freq[li], l.kv_norm, c.norm_eps, l.attn_scale, q->st, qp, qa,
-		    (uint16_t *)q->cache[li]);
+		    (uint16_t *)q->cache[li], (int)expand);
 	else
 		seq_latent_prep_kernel<float><<<n, SEQ_THREADS, rot_lds, q->stream>>>(
 		    q->Z, zin, H, D, R, rk, l.rot_dims, q->rot_freq[li], l.kv_norm, c.norm_eps, l.attn_scale, q->st, qp, qa,
-		    (float *)q->cache[li]);
+		    (float *)q->cache[li], (int)expand);
 	HIPCHK(hipGetLastError());
-	{ // columns [0, kv_rank) of head h's query: W_uk[h]^T q_plain[h], per head [n][dim] x [rank][dim]^T
-		GemmArgs a = plain(qp, H * D, l.w_ukt, D, qa, H * KR, n, rk, D);
-		a.a_bs = D;
-		a.w_bs = (long)rk * D;
-		a.c_bs = KR;
-		TRY(gemm(q, a, H));
-	}
 	AttnArgs a;
 	a.H = H;
-	a.G = 1;
-	a.D = KR;
-	a.V = rk;
-	a.KL = KR;
-	a.VL = KR;
 	a.mask_kind = l.mask_kind;
 	a.mask_size = l.mask_size;
 	a.qk_norm = YALM_QK_NONE;
@@ -951,13 +994,59 @@ static int mixer_latent_direct(Seq *q, int li, int n) {
 	a.q_w = a.k_w = a.temp = a.talk = nullptr;
 	a.eps = c.norm_eps;
 	a.q_mixed = 0;
-	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, qa, nullptr, ctx) : attn_core_t<float>(q, li, n, a, qa, nullptr, ctx));
-	{ // o[h] = W_uv[h] ctx[h]
-		GemmArgs b = plain(ctx, H * rk, l.w_uv, rk, oh, H * V, n, V, rk);
-		b.a_bs = rk;
-		b.w_bs = (long)V * rk;
-		b.c_bs = V;
-		TRY(gemm(q, b, H));
+	if (expand) {
+		const int QH = D + R, NKV = H * (D + V);
+		const float *lat;
+		int ldl;
+		if (bf) { // the cached rows as the product's f32 operand
+			seq_cache_rows_f32_kernel<<<rows, SEQ_THREADS, 0, q->stream>>>((const uint16_t *)q->cache[li], KR, klo, rk, q->ex_c);
+			HIPCHK(hipGetLastError());
+			lat = q->ex_c;
+			ldl = rk;
+		} else {
+			lat = (const float *)q->cache[li] + (size_t)klo * KR;
+			ldl = KR;
+		}
+		TRY(gemm(q, plain(lat, ldl, l.w_ukv, rk, q->ex_kv, NKV, rows, NKV, rk)));
+		if (bf)
+			seq_latent_expand_kernel<uint16_t><<<rows, SEQ_THREADS, 0, q->stream>>>(
+			    q->ex_kv, (const uint16_t *)q->cache[li], klo, H, D, R, V, rk, (uint16_t *)q->ex_k, (uint16_t *)q->ex_v);
+		else
+			seq_latent_expand_kernel<float><<<rows, SEQ_THREADS, 0, q->stream>>>(
+			    q->ex_kv, (const float *)q->cache[li], klo, H, D, R, V, rk, (float *)q->ex_k, (float *)q->ex_v);
+		HIPCHK(hipGetLastError());
+		a.G = H;
+		a.D = QH;
+		a.V = V;
+		a.KL = H * QH;
+		a.VL = H * V;
+		// the attention kernels index rows by position: row klo is the buffers' first
+		const size_t eb = bf ? 2 : 4;
+		const void *kc = (const char *)q->ex_k - (size_t)klo * a.KL * eb;
+		const void *vc = (const char *)q->ex_v - (size_t)klo * a.VL * eb;
+		TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, qa, nullptr, oh, kc, vc)
+		       : attn_core_t<float>(q, li, n, a, qa, nullptr, oh, kc, vc));
+	} else {
+		{ // columns [0, kv_rank) of head h's query: W_uk[h]^T q_plain[h], per head [n][dim] x [rank][dim]^T
+			GemmArgs g = plain(qp, H * D, l.w_ukt, D, qa, H * KR, n, rk, D);
+			g.a_bs = D;
+			g.w_bs = (long)rk * D;
+			g.c_bs = KR;
+			TRY(gemm(q, g, H));
+		}
+		a.G = 1;
+		a.D = KR;
+		a.V = rk;
+		a.KL = KR;
+		a.VL = KR;
+		TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, qa, nullptr, ctx) : attn_core_t<float>(q, li, n, a, qa, nullptr, ctx));
+		{ // o[h] = W_uv[h] ctx[h]
+			GemmArgs b = plain(ctx, H * rk, w_uv, rk, oh, H * V, n, V, rk);
+			b.a_bs = rk;
+			b.w_bs = (long)V * rk;
+			b.c_bs = V;
+			TRY(gemm(q, b, H));
+		}
 	}
 	GemmArgs o = plain(oh, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V);
 	o.bias = l.o_bias;
@@ -1189,6 +1278,7 @@ extern "C" int yalm_seq_step(yalm_seq q, const int *tokens, int n, const int *wa
 		HIPCHK(hipMemcpyAsync(q->tok, tokens + t0, (size_t)m * sizeof(int), hipMemcpyHostToDevice, q->stream));
 		set_step_kernel<<<1, 1, 0, q->stream>>>(q->st, 0, q->host_pos, 0);
 		HIPCHK(hipGetLastError());
+		q->cur_pos = q->host_pos;
 		if (q->dump_on) {
 			if (!q->dump)
 				TRY(sallocT(q, &q->dump, (size_t)c.n_layers * q->cap * c.width));
@@ -1294,6 +1384,7 @@ extern "C" int yalm_seq_time_step(yalm_seq q, int n, int pos0, int iters, float 
 		if (it == 0)
 			(void)hipEventRecord(e0, q->stream);
 		set_step_kernel<<<1, 1, 0, q->stream>>>(q->st, 0, pos0, 0);
+		q->cur_pos = pos0;
 		rc = enqueue_portion(q, q->tok, n);
 		if (rc == YALM_OK)
 			rc = enqueue_logits(q, q->want, 1);

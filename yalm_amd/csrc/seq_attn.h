@@ -250,7 +250,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 // [rank, rank + R) of Qa [t][H][rank + R]: the attention kernels then see H independent heads
 // over ONE key/value head whose key row is the cache row and whose value is its first rank
 // entries. Rotation: the first rot_dims <= R entries in interleaved pairs, as in
-// seq_attn_prep_kernel. Dynamic LDS: max(rot_dims, 2) floats.
+// seq_attn_prep_kernel. expanded != 0 (the portion attends over expanded per-head keys and
+// values, seq_latent_expand_kernel): Qp is not written and Qa is [t][H][D + R], head h's
+// scaled plain part followed by its rotated part. Dynamic LDS: max(rot_dims, 2) floats.
 template <class CT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const float *__restrict__ Z, int ldz, int H, int D,
                                                                       int R, int rank, int rot_dims,
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const floa
                                                                       const float *__restrict__ kv_w, float eps,
                                                                       float scale, const StepState *__restrict__ st,
                                                                       float *__restrict__ Qp, float *__restrict__ Qa,
-                                                                      CT *__restrict__ cache) {
+                                                                      CT *__restrict__ cache, int expanded) {
 	extern __shared__ float rot[];
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x, tid = threadIdx.x;
@@ -295,13 +297,54 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const floa
 		}
 		if (job == 0)
 			cache_store<CT>(crow + rank + d, v);
+		else if (expanded)
+			Qa[((size_t)t * H + job - 1) * QH + D + d] = v * scale;
 		else
 			Qa[((size_t)t * H + job - 1) * KR + rank + d] = v * scale;
 	}
 	for (int i = tid; i < H * D; i += SEQ_THREADS) {
 		const int h = i / D, d = i - h * D;
-		Qp[(size_t)t * H * D + i] = z[(size_t)h * QH + d] * scale;
+		const float v = z[(size_t)h * QH + d] * scale;
+		if (expanded)
+			Qa[((size_t)t * H + h) * QH + d] = v;
+		else
+			Qp[(size_t)t * H * D + i] = v;
 	}
+}
+
+// out[r][c] = cache[row0 + r][c], c < ncols, as f32: cached latent rows as the A operand of the
+// product that expands them.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_cache_rows_f32_kernel(const uint16_t *__restrict__ cache, int row_len,
+                                                                         int row0, int ncols,
+                                                                         float *__restrict__ out) {
+	const int r = blockIdx.x;
+	const uint16_t *src = cache + (size_t)(row0 + r) * row_len;
+	for (int c = threadIdx.x; c < ncols; c += SEQ_THREADS)
+		out[(size_t)r * ncols + c] = bf2f(src[c]);
+}
+
+// Per-head keys and values of the cached positions row0 .. row0 + gridDim.x - 1, from KV [r][H D
+// | H V] (the latent rows times the stacked key and value up-projections) and the cache's
+// rotated key part: Kx [r][H][D + R] = [plain key of head h | the shared rotated part], Vx
+// [r][H][V], in the cache's type. The softmax-attention kernels then see H key/value heads.
+template <class CT>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_latent_expand_kernel(const float *__restrict__ KV,
+                                                                        const CT *__restrict__ cache, int row0, int H,
+                                                                        int D, int R, int V, int rank,
+                                                                        CT *__restrict__ Kx, CT *__restrict__ Vx) {
+	const int r = blockIdx.x, QH = D + R;
+	const float *kv = KV + (size_t)r * H * (D + V);
+	const CT *kr = cache + (size_t)(row0 + r) * (rank + R) + rank;
+	CT *kx = Kx + (size_t)r * H * QH, *vx = Vx + (size_t)r * H * V;
+	for (int i = threadIdx.x; i < H * QH; i += SEQ_THREADS) {
+		const int h = i / QH, d = i - h * QH;
+		if (d < D)
+			cache_store<CT>(kx + i, kv[h * D + d]);
+		else
+			kx[i] = kr[d - D];
+	}
+	for (int i = threadIdx.x; i < H * V; i += SEQ_THREADS)
+		cache_store<CT>(vx + i, kv[H * D + i]);
 }
 
 // ------------------------------------------------------------------ attention, f32 FMA form
@@ -550,12 +593,14 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 // ------------------------------------------------------------------ attention, single token
 // One decoded token: nothing is staged through LDS but the queries. A workgroup owns one key
 // split (gridDim.x = S) of the heads of one key/value head (gridDim.y = G; with score mixing
-// their mixed queries meet the whole key row); a lane owns a key and reads its cache row itself, 16 bytes at a time,
+// their mixed queries meet the whole key row), or of a block of SA_DEC_HB of them (gridDim.z > 1:
+// many heads over one key/value head); a lane owns a key and reads its cache row itself, 16 bytes at a time,
 // eight loads in flight; wave w takes a quarter of the key entries against every head's
 // queries (LDS broadcasts) and leaves partial scores in LDS; wave w then adds them up and
 // normalises heads w, w + 4, ...; then every thread sums NA4 groups of 4 value entries of one
 // head straight from the value rows. Partial results per split as in
 // seq_attn_kernel (S == 1 writes Ctx).
+#define SA_DEC_HB 16
 template <class CT, int NA4>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const float *__restrict__ Q,
                                                                       const CT *__restrict__ Kc,
@@ -569,7 +614,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const floa
 	constexpr int HP = 16;                        // heads per pass over a key slice
 	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
 	const bool talk = a.talk != nullptr;
-	const int Hb = rep, h0 = blockIdx.y * rep; // the heads of one key/value head
+	// the heads of one key/value head (a block of them with gridDim.z > 1)
+	const int hz = gridDim.z > 1 ? blockIdx.z * SA_DEC_HB : 0;
+	const int Hb = gridDim.z > 1 ? min(SA_DEC_HB, rep - hz) : rep, h0 = blockIdx.y * rep + hz;
 	const int DK = talk ? G * D : D, KL = a.KL, VL = a.VL, kcol = talk ? 0 : blockIdx.y * D;
 	const int DK8 = (DK + 7) & ~7, V4n = (V + 3) >> 2;
 	float *qs = lds;               // [Hb][DK8]

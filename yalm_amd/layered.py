@@ -164,7 +164,10 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
         if l.kv_from < 0:
             out["kv_norm"] = ((l.kv_rank,), "f")
         out["w_ukt"] = ((l.heads, l.kv_rank, l.dim), "w")
-        out["w_uv"] = ((l.heads * l.vdim, l.kv_rank), "w")
+        if l.q_rank:
+            out["w_uv"] = ((l.heads * l.vdim, l.kv_rank), "w")
+        else:  # key and value up-projections stacked; the value rows serve as w_uv
+            out["w_ukv"] = ((l.heads * (l.dim + l.vdim), l.kv_rank), "w")
     elif l.mixer == MIX_RGLRU:
         bs = l.rec_width // l.blocks
         out.update(
@@ -698,7 +701,7 @@ def mirorax_pack(c: LayeredConfig, t: dict, cfg: dict = None) -> dict:
             d.update(in_bias=b, o_bias=f(x + "o.b"))
         else:
             d["w_in"] = w(x + "q", x + "dkv")
-            d.update(kv_norm=f(x + "dkv.norm"), sink_w=f(x + "sink"), w_uv=w(x + "uv"))
+            d.update(kv_norm=f(x + "dkv.norm"), sink_w=f(x + "sink"), w_ukv=w(x + "uk", x + "uv"))
             uk = _as_weight(t[x + "uk"], dt).reshape(l.heads, l.dim, l.kv_rank)
             d["w_ukt"] = np.ascontiguousarray(uk.transpose(0, 2, 1))
         d["w_o"] = w(x + "o")

@@ -145,7 +145,7 @@ class SeqLayer(ctypes.Structure):
     PTRS = ("norm1", "norm1b", "norm2", "norm2b", "ls1", "ls2", "pre_add", "sink_w", "o_bias", "router_bias",
             "q_norm", "kv_norm", "in_bias", "head_temp", "talk", "conv_w", "conv_b", "gate_a",
             "gate_a_b", "gate_i", "gate_i_b", "lam", "a_log", "dt_bias", "out_norm", "router", "shared_sg",
-            "w_in", "w_uq", "w_ukt", "w_uv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
+            "w_in", "w_uq", "w_ukt", "w_uv", "w_ukv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
     _fields_ = (
         [(n, c_int) for n in INTS] + [("attn_scale", c_float), ("rec_width", c_int), ("blocks", c_int), ("conv", c_int),
                                       ("ff_kind", c_int), ("ff", c_int), ("experts", c_int), ("top", c_int),
