@@ -79,7 +79,7 @@ def parse():
                          "(Sinulorn-shaped stacks, random bf16 weights) at a few real layer sizes, each beside a "
                          "Llama-shaped decoder of equal width, depth and feed-forward size; one JSON line")
     ap.add_argument("--layered-sizes", default="1024,2048,4096", help="model widths of the --layered legs")
-    ap.add_argument("--layered-design", default="sinulorn", choices=["sinulorn", "lenuzen"],
+    ap.add_argument("--layered-design", default="sinulorn", choices=["sinulorn", "lenuzen", "mirorax"],
                     help="which layer-list design the --layered stack is shaped like")
     return ap.parse_args()
 
@@ -551,6 +551,33 @@ def lenuzen_stack(Ly, M, width, max_tokens):
                             logit_scale=0.7, tied_head=True)
 
 
+def mirorax_stack(Ly, M, width, max_tokens):
+    """A Mirorax-shaped stack at a real layer size, six layer runs: [latent attention + clamped
+    dense feed-forward, gated attention + routed experts] walked twice with the same weights,
+    then gated attention + dense, latent attention + experts. Head size 128; the latent
+    attention with 64 rotated entries, latent rank 512 and a window of 1024; the gated attention
+    with four query heads per key/value head; dense hidden size 3.5 x width, experts whose
+    active hidden size (top x expert + shared) equals it."""
+    heads = width // 128
+    ff = width * 7 // 2
+    dense = dict(ff_kind=Ly.FF_DENSE, ff=ff, limit=7.0, ff_act=Ly.ACT_CLAMP)
+    moe = dict(ff_kind=Ly.FF_MOE, ff=ff // 8, experts=16, top=4, shared_ff=ff // 2, shared_gated=False, ff_act=Ly.ACT_SILU,
+               router_kind=Ly.ROUTER_TOP_SOFTMAX, router_biased=True)
+    lat = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=0, attn_scale=192 ** -0.5,
+               mask_kind=Ly.MASK_WINDOW, mask_size=1024, rot_dims=64, rot_base=10000.0, sink=1, sink_learned=True)
+    att = dict(heads=heads, kv_heads=max(heads // 4, 1), dim=128, vdim=128, attn_scale=128 ** -0.5, mask_kind=Ly.MASK_CAUSAL,
+               out_gate=Ly.GATE_ELEMENT, in_biased=True, o_biased=True)
+    L = Ly.LayerSpec
+    layers = [
+        L(Ly.MIX_LATENT, pre_added=True, **lat, **dense), L(Ly.MIX_ATTN, **att, **moe),
+        L(Ly.MIX_LATENT, pre_added=True, shares=0, **lat, **dense), L(Ly.MIX_ATTN, shares=1, **att, **moe),
+        L(Ly.MIX_ATTN, **att, **dense), L(Ly.MIX_LATENT, **lat, **moe),
+    ]
+    return Ly.LayeredConfig("Mirorax", width, 32000, layers, embed_scale=1.0, norm_eps=1e-6, max_tokens=max_tokens,
+                            weight_dtype=M.BF16, norm_kind=Ly.NORM_RMS, pre_norm=True, pos_embed=False,
+                            block_kind=Ly.BLOCK_PARALLEL)
+
+
 def layered_bench(args, out_file):
     """--layered: tokens/s of a prompt portion (n = 2048 at position 0) and of single-token
     decoding (the device greedy loop at context ~1024) for the layer-list engine, and for a
@@ -564,7 +591,8 @@ def layered_bench(args, out_file):
     n_pf, ctx, steps = 2048, 1024, max(args.steps if args.steps != 256 else 64, 8)
     legs = []
     for width in [int(x) for x in args.layered_sizes.split(",")]:
-        cfg = (lenuzen_stack if args.layered_design == "lenuzen" else layered_stack)(Ly, M, width, n_pf + 64)
+        make = {"lenuzen": lenuzen_stack, "mirorax": mirorax_stack}.get(args.layered_design, layered_stack)
+        cfg = make(Ly, M, width, n_pf + 64)
         model = runtime.SeqModel.synthetic(cfg, seed=3)
         dec = runtime.SeqDecoder(model)
         pf_ms = dec.time_step(n_pf, 0, max(args.prefill_iters, 1))

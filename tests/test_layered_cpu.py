@@ -296,11 +296,14 @@ def test_bench_stacks_are_valid_layer_list_configurations():
     import bench
 
     for width in (1024, 2048, 4096):
-        for make in (bench.layered_stack, bench.lenuzen_stack):
+        for make in (bench.layered_stack, bench.lenuzen_stack, bench.mirorax_stack):
             c = make(Ly, M, width, 2112)
             assert c.width == width and len(c.layers) == 6
             for l in c.layers:
                 shapes = Ly.packed_shapes(c, l)
+                if l.shares >= 0:  # a repeated run of a loop owns its pre_add only
+                    assert set(shapes) <= {"pre_add"} and c.layers[l.shares].mixer == l.mixer
+                    continue
                 assert shapes["w_in"][0] == (l.in_rows, width) and shapes["w_o"][0] == (width, l.mix_out)
                 if l.mixer == Ly.MIX_ATTN:
                     assert l.heads % l.kv_heads == 0 and l.rot_dims <= l.dim

@@ -535,7 +535,7 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 	const bool single = !a.W2 && (a.epi == EPI_NONE || a.epi == EPI_GELU);
 	const int n_big = pair ? (a.N % 64 == 0 ? a.N : 0) : (single ? a.N & ~127 : 0);
 	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.rows && !a.w_sel && a.z_split == 0 && a.ldw == a.K &&
-	    a.K % 64 == 0 && n_big > 0 && a.N - n_big <= 64) {
+	    a.K % 64 == 0 && n_big > 0 && (a.N - n_big <= 64 || (!pair && a.N - n_big < 128))) {
 		const size_t n8 = (size_t)a.M * (a.K / 8);
 		seq_to_bf16_kernel<<<(unsigned)std::min<size_t>((n8 + SEQ_THREADS - 1) / SEQ_THREADS, 4096), SEQ_THREADS, 0,
 		                     q->stream>>>(a.A, a.lda, a.M, a.K, q->a16);
@@ -545,6 +545,15 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 		                            a.epi == EPI_GLU_GELU ? 1 : (a.epi == EPI_GLU_CLAMP ? 2 : 3), a.limit, q->stream)
 		         : pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, n_big, a.C, a.ldc, a.bias,
 		                        a.epi == EPI_GELU ? 1 : 0, q->stream);
+		if (rc == YALM_OK && !pair && n_big < a.N && a.N >= 128) {
+			// the last 128 columns as one more large tile: it computes the columns below n_big a
+			// second time (the same kernel on the same operands: the same values) and the tail
+			const int c0 = a.N - 128;
+			const int rc2 = pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W + (size_t)c0 * a.ldw, 128, a.C + c0,
+			                             a.ldc, a.bias ? a.bias + c0 : nullptr, a.epi == EPI_GELU ? 1 : 0, q->stream);
+			if (rc2 != YALM_ERR_UNSUPPORTED)
+				return rc2;
+		}
 		if (rc == YALM_OK && n_big < a.N) {
 			GemmArgs t = a;
 			t.W = (const uint16_t *)a.W + (size_t)n_big * a.ldw;
@@ -786,26 +795,41 @@ static int attn_mfma_launch(Seq *q, const void *kc, const void *vc, int n, const
 // keys and values whose pointer is moved back by the first row's position)
 template <class CT>
 static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx,
-                       const void *kc = nullptr, const void *vc = nullptr) {
+                       const void *kc = nullptr, const void *vc = nullptr, const float *gate_e = nullptr, int ldg = 0) {
 	if (!kc) {
 		kc = q->cache[li];
 		vc = q->vcache[li];
 	}
+	// gate_e: elementwise gate logits [t][ldg], head h's at column h V: applied by the split merge
+	// where there is one, else by a launch of its own after the attention
+	auto gate_after = [&]() {
+		if (gate_e)
+			seq_gate_mul_kernel<<<dim3(cdiv(a.H * a.V, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(ctx, a.H * a.V, gate_e,
+			                                                                                      ldg, 0, a.H * a.V);
+		HIPCHK(hipGetLastError());
+		return (int)YALM_OK;
+	};
 	const bool talk = a.talk != nullptr;
 	const int DK = talk ? a.G * a.D : a.D;
 	if (sizeof(CT) == 2 && n > GEMV_MAX_M && DK <= 512 && a.V <= 128) { // portions over bf16 caches: the MFMA form
 		const int ks = cdiv(DK, 32);
-		if (ks <= 1) return attn_mfma_launch<1>(q, kc, vc, n, a, Q, gate, ctx);
-		if (ks <= 2) return attn_mfma_launch<2>(q, kc, vc, n, a, Q, gate, ctx);
-		if (ks <= 4) return attn_mfma_launch<4>(q, kc, vc, n, a, Q, gate, ctx);
-		if (ks <= 8) return attn_mfma_launch<8>(q, kc, vc, n, a, Q, gate, ctx);
-		return attn_mfma_launch<16>(q, kc, vc, n, a, Q, gate, ctx);
+		if (ks <= 1) TRY(attn_mfma_launch<1>(q, kc, vc, n, a, Q, gate, ctx));
+		else if (ks <= 2) TRY(attn_mfma_launch<2>(q, kc, vc, n, a, Q, gate, ctx));
+		else if (ks <= 4) TRY(attn_mfma_launch<4>(q, kc, vc, n, a, Q, gate, ctx));
+		else if (ks <= 8) TRY(attn_mfma_launch<8>(q, kc, vc, n, a, Q, gate, ctx));
+		else TRY(attn_mfma_launch<16>(q, kc, vc, n, a, Q, gate, ctx));
+		return gate_after();
 	}
 	const int Hb = a.H / a.G, Gb = talk ? a.G : 1, V4n = (a.V + 3) / 4, D4 = (a.D + 3) & ~3;
 	const CT *Kc = (const CT *)kc, *Vc = (const CT *)vc;
 	const int rep = a.H / a.G;
-	// many heads over one key/value head: blocks of SA_DEC_HB heads per workgroup
-	const int hz = !talk && rep > SA_DEC_HB ? cdiv(rep, SA_DEC_HB) : 1, hb = hz > 1 ? SA_DEC_HB : rep;
+	// many heads over few key/value heads: blocks of heads per workgroup, at most 16 heads each
+	// and small enough that key splits x key/value heads x blocks fill half the chip
+	int hb = rep;
+	if (!talk)
+		while (hb > 1 && (hb > 16 || (rep >= 8 && (long)q->attn_splits[li] * a.G * cdiv(rep, hb) < 128)))
+			hb = (hb + 1) / 2;
+	const int hz = cdiv(rep, hb);
 	const size_t dec_lds = sa_decode_lds_bytes(hb, DK, talk ? a.H * a.D : 0, a.H);
 	if (n == 1 && !a.q_mixed && dec_lds <= 96 * 1024) { // a decoded token: lanes read the cache rows themselves
 		const int S = q->attn_splits[li];
@@ -821,7 +845,8 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 			attr_set = true;                                                                                           \
 		}                                                                                                              \
 		seq_attn_decode_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, Kc, Vc, a, q->st,                        \
-		                                                                   S == 1 ? gate : nullptr, ctx, q->att_part); \
+		                                                                   S == 1 ? gate : nullptr, ctx, q->att_part, \
+		                                                                   hz > 1 ? hb : 0);                           \
 	} while (0)
 		if (na <= 1) SD_LAUNCH(1);
 		else if (na <= 2) SD_LAUNCH(2);
@@ -829,10 +854,12 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 		else if (na <= 8) SD_LAUNCH(8);
 		else SD_LAUNCH(16);
 #undef SD_LAUNCH
-		if (S > 1)
-			seq_latent_merge_kernel<<<a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate);
-		HIPCHK(hipGetLastError());
-		return YALM_OK;
+		if (S > 1) {
+			seq_latent_merge_kernel<<<a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate, gate_e, ldg, a.H);
+			HIPCHK(hipGetLastError());
+			return YALM_OK;
+		}
+		return gate_after();
 	}
 	// tokens per workgroup: up to 32 rows, their queries within 64 KB of LDS
 	int TQ = std::max(1, std::min(32 / Hb, n));
@@ -864,10 +891,12 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 	else if (na <= 8) SA_LAUNCH(8);
 	else SA_LAUNCH(16);
 #undef SA_LAUNCH
-	if (S > 1)
-		seq_latent_merge_kernel<<<n * a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate);
-	HIPCHK(hipGetLastError());
-	return YALM_OK;
+	if (S > 1) {
+		seq_latent_merge_kernel<<<n * a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate, gate_e, ldg, a.H);
+		HIPCHK(hipGetLastError());
+		return YALM_OK;
+	}
+	return gate_after();
 }
 
 // Softmax attention over cached keys and values: one input projection (queries, keys, values,
@@ -926,12 +955,9 @@ static int mixer_attn(Seq *q, int li, int n) {
 		    (const float *)l.w_in + (size_t)zmain * c.width, gbias);
 	HIPCHK(hipGetLastError());
 	const float *gp = a.out_gate ? gate : nullptr;
-	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, Q, gp, ctx) : attn_core_t<float>(q, li, n, a, Q, gp, ctx));
-	if (l.out_gate == 2) {
-		seq_gate_mul_kernel<<<dim3(cdiv(H * V, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(ctx, H * V, q->Z, zin, zin - H * V,
-		                                                                                   H * V);
-		HIPCHK(hipGetLastError());
-	}
+	const float *ge = l.out_gate == 2 ? q->Z + (zin - H * V) : nullptr; // elementwise gate logits close the Z rows
+	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, Q, gp, ctx, nullptr, nullptr, ge, zin)
+	       : attn_core_t<float>(q, li, n, a, Q, gp, ctx, nullptr, nullptr, ge, zin));
 	GemmArgs o = plain(ctx, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V);
 	o.bias = l.o_bias;
 	return gemm(q, o);
@@ -1154,10 +1180,19 @@ static int par_close(Seq *q, int li, int n) {
 	const bool moe = l.ff_kind == YALM_FF_MOE;
 	const bool gated = moe && l.shared_ff > 0 && l.shared_sg;
 	float *dump = q->dump_on && q->dump ? q->dump + (size_t)li * n * c.width : nullptr;
-	seq_par_close_kernel<<<n, SEQ_THREADS, (size_t)c.width * sizeof(float), q->stream>>>(
-	    q->X, q->Y, l.ls1, (l.ff_kind != YALM_FF_NONE && !moe) ? q->Y2 : nullptr, l.ls2, moe ? q->B[1] : nullptr, q->wt,
-	    moe ? l.top : 0, moe && l.shared_ff > 0 ? q->B[3] : nullptr, gated ? q->sgate : nullptr, dump,
-	    nx ? nx->pre_add : nullptr, c.norm_eps, c.width, nx ? nx->norm1 : nullptr, q->Hn, (int)q->ln);
+#define PC_ARGS                                                                                                        \
+	q->X, q->Y, l.ls1, (l.ff_kind != YALM_FF_NONE && !moe) ? q->Y2 : nullptr, l.ls2, moe ? q->B[1] : nullptr, q->wt,    \
+	    moe ? l.top : 0, moe && l.shared_ff > 0 ? q->B[3] : nullptr, gated ? q->sgate : nullptr, dump,                 \
+	    nx ? nx->pre_add : nullptr, c.norm_eps, c.width, nx ? nx->norm1 : nullptr, q->Hn, (int)q->ln
+	if (c.width <= 4 * SEQ_THREADS)
+		seq_par_close_reg_kernel<4><<<n, SEQ_THREADS, 0, q->stream>>>(PC_ARGS);
+	else if (c.width <= 8 * SEQ_THREADS)
+		seq_par_close_reg_kernel<8><<<n, SEQ_THREADS, 0, q->stream>>>(PC_ARGS);
+	else if (c.width <= 16 * SEQ_THREADS)
+		seq_par_close_reg_kernel<16><<<n, SEQ_THREADS, 0, q->stream>>>(PC_ARGS);
+	else
+		seq_par_close_kernel<<<n, SEQ_THREADS, (size_t)c.width * sizeof(float), q->stream>>>(PC_ARGS);
+#undef PC_ARGS
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
 }

@@ -593,21 +593,22 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 // ------------------------------------------------------------------ attention, single token
 // One decoded token: nothing is staged through LDS but the queries. A workgroup owns one key
 // split (gridDim.x = S) of the heads of one key/value head (gridDim.y = G; with score mixing
-// their mixed queries meet the whole key row), or of a block of SA_DEC_HB of them (gridDim.z > 1:
-// many heads over one key/value head); a lane owns a key and reads its cache row itself, 16 bytes at a time,
+// their mixed queries meet the whole key row), or of a block of hblk of them (hblk > 0, gridDim.z
+// blocks: many heads over one key/value head, where key splits alone are too few workgroups to
+// fill the chip); a lane owns a key and reads its cache row itself, 16 bytes at a time,
 // eight loads in flight; wave w takes a quarter of the key entries against every head's
 // queries (LDS broadcasts) and leaves partial scores in LDS; wave w then adds them up and
 // normalises heads w, w + 4, ...; then every thread sums NA4 groups of 4 value entries of one
 // head straight from the value rows. Partial results per split as in
 // seq_attn_kernel (S == 1 writes Ctx).
-#define SA_DEC_HB 16
 template <class CT, int NA4>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const float *__restrict__ Q,
                                                                       const CT *__restrict__ Kc,
                                                                       const CT *__restrict__ Vc, AttnArgs a,
                                                                       const StepState *__restrict__ st,
                                                                       const float *__restrict__ gate,
-                                                                      float *__restrict__ Ctx, float *__restrict__ part) {
+                                                                      float *__restrict__ Ctx, float *__restrict__ part,
+                                                                      int hblk) {
 	extern __shared__ __attribute__((aligned(16))) float lds[];
 	constexpr int NW = SEQ_THREADS / 64;
 	constexpr int EPL = sizeof(CT) == 2 ? 8 : 4; // cache entries per 16-byte load
@@ -615,8 +616,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const floa
 	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
 	const bool talk = a.talk != nullptr;
 	// the heads of one key/value head (a block of them with gridDim.z > 1)
-	const int hz = gridDim.z > 1 ? blockIdx.z * SA_DEC_HB : 0;
-	const int Hb = gridDim.z > 1 ? min(SA_DEC_HB, rep - hz) : rep, h0 = blockIdx.y * rep + hz;
+	const int hz = hblk > 0 ? blockIdx.z * hblk : 0;
+	const int Hb = hblk > 0 ? min(hblk, rep - hz) : rep, h0 = blockIdx.y * rep + hz;
 	const int DK = talk ? G * D : D, KL = a.KL, VL = a.VL, kcol = talk ? 0 : blockIdx.y * D;
 	const int DK8 = (DK + 7) & ~7, V4n = (V + 3) >> 2;
 	float *qs = lds;               // [Hb][DK8]

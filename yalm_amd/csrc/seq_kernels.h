@@ -385,6 +385,94 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__res
 		Hn[(size_t)t * n + i] = (row[i] - mu) * r * w_next[i];
 }
 
+// The same seam with the row in registers (rows of up to E * SEQ_THREADS entries): every
+// operand row and vector is loaded at once, one memory round trip instead of one per pass.
+template <int E>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_reg_kernel(float *__restrict__ X, const float *__restrict__ Y1,
+                                                                        const float *__restrict__ s1,
+                                                                        const float *__restrict__ Y2,
+                                                                        const float *__restrict__ s2,
+                                                                        const float *__restrict__ Yx,
+                                                                        const float *__restrict__ wt, int top,
+                                                                        const float *__restrict__ Ys,
+                                                                        const float *__restrict__ sgate,
+                                                                        float *__restrict__ dump,
+                                                                        const float *__restrict__ add, float eps, int n,
+                                                                        const float *__restrict__ w_next,
+                                                                        float *__restrict__ Hn, int ln) {
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x;
+	float x[E], y1[E], a1[E], f[E], a2[E], ad[E], wn[E];
+	const bool ff = Yx || Y2;
+#pragma unroll
+	for (int e = 0; e < E; ++e) {
+		const int i = threadIdx.x + e * SEQ_THREADS;
+		const bool in = i < n;
+		x[e] = in ? X[(size_t)t * n + i] : 0.0f;
+		y1[e] = in ? Y1[(size_t)t * n + i] : 0.0f;
+		a1[e] = in ? s1[i] : 0.0f;
+		a2[e] = (in && ff) ? s2[i] : 0.0f;
+		ad[e] = (in && add) ? add[i] : 0.0f;
+		wn[e] = (in && w_next) ? w_next[i] : 0.0f;
+		f[e] = (in && Y2 && !Yx) ? Y2[(size_t)t * n + i] : 0.0f;
+	}
+	if (Yx) {
+		for (int k = 0; k < top; ++k) {
+			const float w = wt[(size_t)t * top + k];
+#pragma unroll
+			for (int e = 0; e < E; ++e) {
+				const int i = threadIdx.x + e * SEQ_THREADS;
+				f[e] = fmaf(w, i < n ? Yx[((size_t)t * top + k) * n + i] : 0.0f, f[e]);
+			}
+		}
+		if (Ys) {
+			const float w = sgate ? sgate[t] : 1.0f;
+#pragma unroll
+			for (int e = 0; e < E; ++e) {
+				const int i = threadIdx.x + e * SEQ_THREADS;
+				f[e] = fmaf(w, i < n ? Ys[(size_t)t * n + i] : 0.0f, f[e]);
+			}
+		}
+	}
+	float ss = 0.0f, sm = 0.0f;
+#pragma unroll
+	for (int e = 0; e < E; ++e) {
+		const int i = threadIdx.x + e * SEQ_THREADS;
+		float v = fmaf(a1[e], y1[e], x[e]);
+		if (ff)
+			v = fmaf(a2[e], f[e], v);
+		if (dump && i < n)
+			dump[(size_t)t * n + i] = v;
+		v += ad[e];
+		x[e] = v;
+		if (i < n) {
+			X[(size_t)t * n + i] = v;
+			ss = fmaf(v, v, ss);
+			sm += v;
+		}
+	}
+	if (!w_next)
+		return;
+	if (ln) {
+		const float mu = block_sum(sm, red) / (float)n;
+		ss = 0.0f;
+#pragma unroll
+		for (int e = 0; e < E; ++e)
+			if (threadIdx.x + e * SEQ_THREADS < n) {
+				x[e] -= mu;
+				ss = fmaf(x[e], x[e], ss);
+			}
+	}
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll
+	for (int e = 0; e < E; ++e) {
+		const int i = threadIdx.x + e * SEQ_THREADS;
+		if (i < n)
+			Hn[(size_t)t * n + i] = x[e] * r * wn[e];
+	}
+}
+
 // C[t][j] *= sigmoid(Z[t][col0 + j]), j < n: an elementwise output gate whose logits are
 // columns of the input projection's result.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_gate_mul_kernel(float *__restrict__ C, int ldc,
@@ -1571,10 +1659,13 @@ static inline size_t att_lds_bytes(int rank) {
 	return sizeof(float) * ((size_t)ATT_BR * r4 + (size_t)ATT_KT * (r4 + 4) + ATT_BR * ATT_KT + 3 * ATT_BR);
 }
 // Ctx[r] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits of row r
-// (times gate[r] if given).
+// (times gate[r] if given; gate_e: times sigmoid of the row's own gate logits, row r = token
+// r / H, head r % H, logits at gate_e[token * ldg + head * rank + d]).
 __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__restrict__ part, int S, int rank,
                                                               float *__restrict__ Ctx,
-                                                              const float *__restrict__ gate = nullptr) {
+                                                              const float *__restrict__ gate = nullptr,
+                                                              const float *__restrict__ gate_e = nullptr, int ldg = 0,
+                                                              int H = 1) {
 	__shared__ float wsm[64]; // S <= 64: lane s holds split s
 	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4, lane = threadIdx.x;
 	const float *pp = part + (size_t)r * S * stride;
@@ -1590,6 +1681,8 @@ __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__res
 #pragma unroll 4
 		for (int s = 0; s < S; ++s)
 			v = fmaf(wsm[s], pp[(size_t)s * stride + d], v);
+		if (gate_e)
+			v *= sq_sigmoid(gate_e[(size_t)(r / H) * ldg + (size_t)(r % H) * rank + d]);
 		Ctx[(size_t)r * rank + d] = v;
 	}
 }
