@@ -611,7 +611,7 @@ static int attn_t(Seq *q, const float *Qa, const void *cache, int rank, int H, i
 	else ATT_LAUNCH(4);
 #undef ATT_LAUNCH
 	if (S > 1)
-		seq_latent_merge_kernel<<<NR, 64, 0, q->stream>>>(q->att_part, S, rank, ctx);
+		seq_latent_merge_kernel<<<NR, SEQ_THREADS, 0, q->stream>>>(q->att_part, S, rank, ctx);
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
 }
@@ -855,7 +855,7 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 		else SD_LAUNCH(16);
 #undef SD_LAUNCH
 		if (S > 1) {
-			seq_latent_merge_kernel<<<a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate, gate_e, ldg, a.H);
+			seq_latent_merge_kernel<<<a.H, SEQ_THREADS, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate, gate_e, ldg, a.H);
 			HIPCHK(hipGetLastError());
 			return YALM_OK;
 		}
@@ -892,7 +892,7 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 	else SA_LAUNCH(16);
 #undef SA_LAUNCH
 	if (S > 1) {
-		seq_latent_merge_kernel<<<n * a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate, gate_e, ldg, a.H);
+		seq_latent_merge_kernel<<<n * a.H, SEQ_THREADS, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate, gate_e, ldg, a.H);
 		HIPCHK(hipGetLastError());
 		return YALM_OK;
 	}
@@ -995,12 +995,13 @@ static int mixer_latent_direct(Seq *q, int li, int n) {
 	const bool expand = l.w_ukv && n > 1 && rows <= q->ex_rows && (n >= 32 || !absorbed_ok);
 	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
 	const size_t rot_lds = (size_t)std::max(l.rot_dims, 2) * sizeof(float);
+	const dim3 pg(n, n <= GEMV_MAX_M ? 4 : 1); // a few tokens: each token's work spread over four workgroups
 	if (bf)
-		seq_latent_prep_kernel<uint16_t><<<n, SEQ_THREADS, rot_lds, q->stream>>>(
+		seq_latent_prep_kernel<uint16_t><<<pg, SEQ_THREADS, rot_lds, q->stream>>>(
 		    q->Z, zin, H, D, R, rk, l.rot_dims, q->rot_freq[li], l.kv_norm, c.norm_eps, l.attn_scale, q->st, qp, qa,
 		    (uint16_t *)q->cache[li], (int)expand);
 	else
-		seq_latent_prep_kernel<float><<<n, SEQ_THREADS, rot_lds, q->stream>>>(
+		seq_latent_prep_kernel<float><<<pg, SEQ_THREADS, rot_lds, q->stream>>>(
 		    q->Z, zin, H, D, R, rk, l.rot_dims, q->rot_freq[li], l.kv_norm, c.norm_eps, l.attn_scale, q->st, qp, qa,
 		    (float *)q->cache[li], (int)expand);
 	HIPCHK(hipGetLastError());

@@ -252,7 +252,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 // entries. Rotation: the first rot_dims <= R entries in interleaved pairs, as in
 // seq_attn_prep_kernel. expanded != 0 (the portion attends over expanded per-head keys and
 // values, seq_latent_expand_kernel): Qp is not written and Qa is [t][H][D + R], head h's
-// scaled plain part followed by its rotated part. Dynamic LDS: max(rot_dims, 2) floats.
+// scaled plain part followed by its rotated part. The workgroups of a token (gridDim.y) share its
+// outputs (each works the rotation table and the latent's rms out for itself). Dynamic LDS:
+// max(rot_dims, 2) floats.
 template <class CT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const float *__restrict__ Z, int ldz, int H, int D,
                                                                       int R, int rank, int rot_dims,
@@ -273,6 +275,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const floa
 		rot[i] = cosf(red_ang);
 		rot[half + i] = sinf(red_ang);
 	}
+	const int i0 = blockIdx.y * SEQ_THREADS + tid, istep = gridDim.y * SEQ_THREADS; // this workgroup's share of every loop
 	const int QH = D + R, QN = H * QH, KR = rank + R;
 	const float *z = Z + (size_t)t * ldz;
 	const float *lat = z + QN;
@@ -281,10 +284,10 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const floa
 		ss = fmaf(lat[i], lat[i], ss);
 	const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)rank + eps); // also orders rot[] before its readers
 	CT *crow = cache + (size_t)p * KR;
-	for (int i = tid; i < rank; i += SEQ_THREADS)
+	for (int i = i0; i < rank; i += istep)
 		cache_store<CT>(crow + i, lat[i] * r * kv_w[i]);
 	// the rotated parts: job 0 is the shared key part, job 1 + h head h's query part
-	for (int i = tid; i < (H + 1) * R; i += SEQ_THREADS) {
+	for (int i = i0; i < (H + 1) * R; i += istep) {
 		const int job = i / R, d = i - job * R;
 		const float *src = job == 0 ? lat + rank : z + (size_t)(job - 1) * QH + D;
 		float v;
@@ -302,7 +305,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_prep_kernel(const floa
 		else
 			Qa[((size_t)t * H + job - 1) * KR + rank + d] = v * scale;
 	}
-	for (int i = tid; i < H * D; i += SEQ_THREADS) {
+	for (int i = i0; i < H * D; i += istep) {
 		const int h = i / D, d = i - h * D;
 		const float v = z[(size_t)h * QH + d] * scale;
 		if (expanded)

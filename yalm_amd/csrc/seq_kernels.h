@@ -1661,13 +1661,16 @@ static inline size_t att_lds_bytes(int rank) {
 // Ctx[r] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits of row r
 // (times gate[r] if given; gate_e: times sigmoid of the row's own gate logits, row r = token
 // r / H, head r % H, logits at gate_e[token * ldg + head * rank + d]).
-__global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__restrict__ part, int S, int rank,
+// One workgroup per row: every wave works the splits' weights out for itself (lane s holds
+// split s, S <= 64), then the waves share the row's entries.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_latent_merge_kernel(const float *__restrict__ part, int S, int rank,
                                                               float *__restrict__ Ctx,
                                                               const float *__restrict__ gate = nullptr,
                                                               const float *__restrict__ gate_e = nullptr, int ldg = 0,
                                                               int H = 1) {
-	__shared__ float wsm[64]; // S <= 64: lane s holds split s
-	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4, lane = threadIdx.x;
+	__shared__ float wsm_all[SEQ_THREADS];
+	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4, lane = threadIdx.x & 63;
+	float *wsm = wsm_all + (threadIdx.x & ~63); // this wave's copy
 	const float *pp = part + (size_t)r * S * stride;
 	const float m = lane < S ? pp[(size_t)lane * stride + rank4] : -FLT_MAX;
 	const float l = lane < S ? pp[(size_t)lane * stride + rank4 + 1] : 0.0f;
@@ -1676,9 +1679,9 @@ __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__res
 	const float inv = (gate ? gate[r] : 1.0f) / wave_sum(w * l);
 	wsm[lane] = w * inv;
 	__syncthreads();
-	for (int d = lane; d < rank; d += 64) {
+	for (int d = threadIdx.x; d < rank; d += SEQ_THREADS) {
 		float v = 0.0f;
-#pragma unroll 4
+#pragma unroll 8
 		for (int s = 0; s < S; ++s)
 			v = fmaf(wsm[s], pp[(size_t)s * stride + d], v);
 		if (gate_e)
