@@ -573,7 +573,7 @@ def mirorax_stack(Ly, M, width, max_tokens):
         L(Ly.MIX_LATENT, pre_added=True, shares=0, **lat, **dense), L(Ly.MIX_ATTN, shares=1, **att, **moe),
         L(Ly.MIX_ATTN, **att, **dense), L(Ly.MIX_LATENT, **lat, **moe),
     ]
-    return Ly.LayeredConfig("Mirorax", width, 32000, layers, embed_scale=1.0, norm_eps=1e-6, max_tokens=max_tokens,
+    return Ly.LayeredConfig("Mirorax", width, 32000, layers, embed_scale=1.0, norm_eps=1e-5, max_tokens=max_tokens,
                             weight_dtype=M.BF16, norm_kind=Ly.NORM_RMS, pre_norm=True, pos_embed=False,
                             block_kind=Ly.BLOCK_PARALLEL)
 
