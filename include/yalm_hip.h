@@ -312,12 +312,14 @@ int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
  * A second decoder kind beside yalm_decoder, for designs whose layers differ from one
  * another: every layer names a token mixer (latent attention over a cached low-rank
  * key/value latent, a real-gated linear recurrence, a gated delta rule, softmax attention
- * over cached keys and values with a window or chunk mask) and a feed-forward (none, dense
+ * over cached keys and values with a window or chunk mask, a selective state-space layer; or
+ * two of them side by side on the same input) and a feed-forward (none, dense
  * GLU, routed experts with an optional shared expert, a plain two-matrix one), each with
  * its own sizes and constants. Serial blocks (block_kind = YALM_BLOCK_SERIAL): around every
  * sublayer x += norm_b(f(norm(x))) (pre_norm = 1) or x += norm_b(f(x)) (pre_norm = 0).
  * Parallel blocks (YALM_BLOCK_PARALLEL): h = norm1(x), x += ls1 * mixer(h) + ls2 * ff(h), one
- * norm read by both sublayers, each result scaled elementwise by its own vector. The norms
+ * norm read by both sublayers, each result scaled elementwise by its own vector (NULL: 1); a
+ * layer of such a block that has norm2 feeds its feed-forward norm2(x) of the same x. The norms
  * are rms norms or mean-subtracting layer norms (norm_kind), both with a weight and no bias.
  * The layer array is the order the layers RUN in: a block of layers that is walked several
  * times with the same weights is passed unrolled, its entries naming the same tensors, and
@@ -331,7 +333,7 @@ int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
  * matrices: YALM_BF16 (bf16 MFMA products with f32 accumulation for portions, bf16
  * weight-streaming GEMVs for single tokens) or YALM_F32 (true f32 products).
  * Matrices are row-major [out][in]. */
-enum { YALM_MIX_LATENT = 0, YALM_MIX_RGLRU = 1, YALM_MIX_DELTA = 2, YALM_MIX_ATTN = 3 };
+enum { YALM_MIX_LATENT = 0, YALM_MIX_RGLRU = 1, YALM_MIX_DELTA = 2, YALM_MIX_ATTN = 3, YALM_MIX_SSM = 4 };
 enum { YALM_FF_NONE = 0, YALM_FF_DENSE = 1, YALM_FF_MOE = 2, YALM_FF_PLAIN = 3 };
 enum { YALM_NORM_RMS = 0, YALM_NORM_LAYER = 1 };
 enum { YALM_BLOCK_SERIAL = 0, YALM_BLOCK_PARALLEL = 1 };
@@ -339,10 +341,14 @@ enum { YALM_BLOCK_SERIAL = 0, YALM_BLOCK_PARALLEL = 1 };
 enum { YALM_ACT_DEFAULT = 0, /* dense: gelu; experts and shared expert: clamp */
 	   YALM_ACT_GELU = 1,  /* gelu_tanh(g) u */
 	   YALM_ACT_CLAMP = 2, /* g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit) */
-	   YALM_ACT_SILU = 3   /* g sigmoid(g) u */ };
+	   YALM_ACT_SILU = 3,  /* g sigmoid(g) u */
+	   YALM_ACT_RELU2 = 4  /* plain feed-forward only: w_down max(w_up x, 0)^2 */ };
 /* routed experts: how the `top` experts and their weights come from the router logits */
 enum { YALM_ROUTER_SOFTMAX_TOP = 0, /* softmax over all experts, best groups, top scores, weight = score * router_scale */
-	   YALM_ROUTER_TOP_SOFTMAX = 1  /* the top logits (+ router_bias) win, weights = softmax over the chosen logits only */ };
+	   YALM_ROUTER_TOP_SOFTMAX = 1, /* the top logits (+ router_bias) win, weights = softmax over the chosen logits only */
+	   YALM_ROUTER_SIGMOID_GROUPS = 2 /* scores sigmoid(logit); the choice ranks score + router_bias: a group by the sum of
+	                                    its two largest, the `top` largest within the groups_keep best groups win (ties: the
+	                                    lower index); weight = score * router_scale (without the bias, not renormalised) */ };
 /* attn: which earlier positions j <= i a position i sees */
 enum { YALM_MASK_CAUSAL = 0, /* all of them */
 	   YALM_MASK_WINDOW = 1, /* i - j < mask_size */
@@ -350,7 +356,10 @@ enum { YALM_MASK_CAUSAL = 0, /* all of them */
 /* attn: norm of queries and keys */
 enum { YALM_QK_NONE = 0,
 	   YALM_QK_HEAD_UNIT = 1, /* after the rotation, every head divided by its rms over dim, no weight */
-	   YALM_QK_WHOLE = 2 /* before the rotation, rms norm over the whole projection with weights q_norm / kv_norm */ };
+	   YALM_QK_WHOLE = 2, /* before the rotation, rms norm over the whole projection with weights q_norm / kv_norm */
+	   YALM_QK_HEAD_W = 3 /* every head rms-normed over dim, times q_norm / kv_norm [dim] shared by all heads (no rotation) */ };
+/* delta: activation of the output gate */
+enum { YALM_GATE_SILU = 0, YALM_GATE_SIGMOID = 1 };
 
 typedef struct yalm_seq_layer {
 	int mixer;                     /* YALM_MIX_* */
@@ -389,6 +398,26 @@ typedef struct yalm_seq_layer {
 	                                  times and the pair that turns rot_slow times within rot_orig positions (f / factor
 	                                  where slower, f where faster, a linear ramp between), cos and sin times
 	                                  0.1 ln(rot_factor) + 1 */
+	/* ssm (YALM_MIX_SSM): heads heads of vdim channels, a state of ssm_state x vdim per head, ssm_groups groups of
+	   B / C vectors (head h reads group h / (heads / ssm_groups)); w_in rows [gate: heads vdim | x: heads vdim |
+	   B: ssm_groups ssm_state | C: the same | step: heads]; x | B | C pass the convolution (conv taps, conv_w,
+	   conv_b) and silu; dt = softplus(step + dt_bias[h]); S <- exp(-exp(a_log[h]) dt) S + dt B x^T; y = S^T C +
+	   d_skip[h] x; y silu(gate) is rms-normed in norm_groups equal parts, times out_norm [heads vdim]; then w_o */
+	int ssm_state, ssm_groups, norm_groups;
+	/* delta: decay_rank > 0: one decay per head and key channel, g = exp(-exp(a_log[h]) softplus(w_a2 (a) + dt_bias)),
+	   `a` the decay_rank decay rows of w_in (instead of heads), w_a2 [heads dim][decay_rank], dt_bias [heads dim];
+	   gate_rank > 0: the output gate's logits are w_g2 (g), `g` the gate_rank gate rows of w_in (instead of heads
+	   vdim), w_g2 [heads vdim][gate_rank]; gate_act: YALM_GATE_* */
+	int decay_rank, gate_rank, gate_act;
+	/* attn: q_temp_every > 0: the query at position p times 1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1) */
+	float q_temp_coef;
+	int q_temp_every;
+	/* attn: rel_rows > 0: rel[bucket(i - j)][h] is added to the scaled score of query i and key j; bucket(n) = n below
+	   rel_rows / 2, else min(rel_rows - 1, rel_rows / 2 + floor(ln(n / (rel_rows / 2)) / ln(rel_max / (rel_rows / 2))
+	   (rel_rows - rel_rows / 2))) (integer halves) */
+	int rel_rows;
+	float rel_max;
+	float join_scale;              /* side != NULL: mixer result = join_scale (rms(a) join_w + rms(b) side_join_w) */
 	/* f32 vectors */
 	const float *norm1, *norm1b, *norm2, *norm2b; /* [width] each; norm2* unused without a feed-forward; parallel blocks: norm1 only */
 	const float *ls1, *ls2;         /* parallel blocks: [width] scales of the mixer's and the feed-forward's result */
@@ -403,13 +432,15 @@ typedef struct yalm_seq_layer {
 	const float *conv_w, *conv_b;   /* [channels][conv] (last column = current token); rglru bias [rec_width] */
 	const float *gate_a, *gate_a_b, *gate_i, *gate_i_b; /* rglru: [blocks][bs][bs], [rec_width] (bs = rec_width / blocks) */
 	const float *lam;               /* rglru: [rec_width] */
-	const float *a_log, *dt_bias, *out_norm; /* delta: [heads], [heads], [vdim] */
+	const float *a_log, *dt_bias, *out_norm; /* delta: [heads], [heads] ([heads dim] with decay_rank), [vdim]; ssm: [heads], [heads], [heads vdim] */
 	const float *router, *shared_sg; /* moe: [experts][width]; [width]: the shared expert times sigmoid(shared_sg . x), NULL: times 1 */
 	/* matrices of weight_dtype */
 	const void *w_in;  /* latent: [q_rank (+ kv_rank if own latent)][width] (query down, latent down), with q_rank = 0
 	                      [heads (dim + rot_dim) + kv_rank + rot_dim][width] (queries, latent down, rotated key part);
 	                      rglru: [2 rec_width][width] (gate branch, recurrent branch);
-	                      delta: [2 kv_heads dim + 2 heads vdim + 2 heads][width] (q, k, v, output gate, beta, decay);
+	                      delta: [2 kv_heads dim + heads vdim + (gate_rank | heads vdim) + heads + (decay_rank | heads)][width]
+	                      (q, k, v, output gate, beta, decay);
+	                      ssm: [2 heads vdim + 2 ssm_groups ssm_state + heads][width] (gate, x, B, C, step);
 	                      attn: [heads dim + kv_heads dim + kv_heads vdim (+ heads | heads vdim if out_gate)][width] (q, k, v, gate) */
 	const void *w_uq;  /* latent: [heads dim][q_rank] (unused with q_rank = 0) */
 	const void *w_ukt; /* latent: [heads][kv_rank][dim], the key up-projection transposed per head */
@@ -421,6 +452,14 @@ typedef struct yalm_seq_layer {
 	const void *w_gate, *w_up, *w_down; /* dense: [ff][width] x2, [width][ff]; moe: the same per expert, stacked;
 	                                       plain: w_down gelu(w_up x), no w_gate */
 	const void *ws_gate, *ws_up, *ws_down; /* moe shared expert */
+	const float *rel;              /* attn: [rel_rows][heads], see rel_rows */
+	const float *d_skip;           /* ssm: [heads] */
+	const float *join_w, *side_join_w; /* side != NULL: [width] each */
+	const void *w_a2, *w_g2;       /* delta: see decay_rank / gate_rank */
+	const struct yalm_seq_layer *side; /* HOST pointer or NULL: a second mixer that reads the same input beside this
+	                                  one (its mixer fields and tensors only; no norms, no feed-forward, no side of its
+	                                  own), with caches and states of its own; the two results are each rms-normed over
+	                                  the width (no mean taken off) and summed, see join_scale */
 } yalm_seq_layer;
 
 typedef struct yalm_seq_config {
@@ -439,6 +478,8 @@ typedef struct yalm_seq_weights {
 	const float *final_norm; /* [width] */
 	const void *head;        /* [vocab][width] */
 	const yalm_seq_layer *layers; /* HOST array of n_layers entries, copied by yalm_seq_create */
+	const float *embed_norm;  /* [width] or NULL: the embedding row (scaled, with its position vector) is normed
+	                             with this weight before it becomes the stream */
 } yalm_seq_weights;
 
 typedef struct yalm_seq_s *yalm_seq;

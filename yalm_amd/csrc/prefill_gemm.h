@@ -114,7 +114,7 @@ struct E16StoreF32 {
 };
 
 // bf16 operands (epi_bf16), C[m][n] = act(acc (+ bias[n])) in f32: the layer-list engine's plain
-// products; act 1: the tanh form of gelu (an ungated feed-forward's first product)
+// products; act 1: the tanh form of gelu, act 2: max(., 0)^2 (an ungated feed-forward's first product)
 struct E16StoreF32B {
 	static constexpr bool NEEDS_LDS = false;
 	static constexpr bool BF16 = true;
@@ -137,6 +137,8 @@ struct E16StoreF32B {
 					float v = acc[i][j][r] + b;
 					if (act == 1)
 						v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+					else if (act == 2)
+						v = fmaxf(v, 0.0f) * fmaxf(v, 0.0f);
 					if (m < M)
 						c[(size_t)m * ldc + n] = v;
 				}

@@ -1,6 +1,7 @@
 // seq.hip — the layer-list engine of the C ABI (include/yalm_hip.h, "layer-list models"):
 // a decoder whose layers each name their token mixer (latent attention, real-gated linear
-// recurrence, gated delta rule, softmax attention with a window or chunk mask) and
+// recurrence, gated delta rule, softmax attention with a window or chunk mask, selective
+// state-space layer, or two of them side by side) and
 // feed-forward (dense GLU, routed experts, plain), holding one sequence's latent and
 // key / value caches and recurrent / convolution states in HBM. One step function
 // serves whole prompts, portions of prompts and single decoded tokens; the device greedy
@@ -43,6 +44,13 @@ struct yalm_seq_s {
 	size_t bw = 0;               // floats per row of the work buffers B0..B3
 	int zw = 0;                  // floats per row of Z (the widest input projection)
 	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Y2 = nullptr, *Z = nullptr, *B[4] = {};
+	float *Hn2 = nullptr;        // parallel blocks whose feed-forward has a norm of its own: norm2(x)
+	float *Y3 = nullptr;         // the result of a layer's second mixer (side) before the two are joined
+	float *Yout = nullptr;       // where the mixer being enqueued leaves its result: Y, or Y3
+	const float *embed_norm = nullptr;
+	std::vector<int> side_of;    // per layer: index in L of its second mixer, or -1 (sides follow the n_layers entries)
+	std::vector<float *> rel_dist; // attn with a distance bias: [rel_far + 1][heads], the bucketed table per distance
+	std::vector<int> rel_far;
 	const float *In = nullptr;   // what a sublayer reads: Hn (pre_norm) or X itself
 	float *Xalt = nullptr, *Xbase = nullptr; // single tokens without opening norms: the stream alternates between two rows
 	const float *pend_wb = nullptr; // a closing norm not yet applied: X += norm(Y) pend_wb, owed to the next product
@@ -113,7 +121,10 @@ static int in_rows(const yalm_seq_layer &l) {
 	case YALM_MIX_ATTN:
 		return l.heads * l.dim + l.kv_heads * (l.dim + l.vdim) +
 		       (l.out_gate == 2 ? l.heads * l.vdim : (l.out_gate ? l.heads : 0));
-	default: return 2 * l.kv_heads * l.dim + 2 * l.heads * l.vdim + 2 * l.heads;
+	case YALM_MIX_SSM: return 2 * l.heads * l.vdim + 2 * l.ssm_groups * l.ssm_state + l.heads;
+	default:
+		return 2 * l.kv_heads * l.dim + l.heads * l.vdim + (l.gate_rank > 0 ? l.gate_rank : l.heads * l.vdim) + l.heads +
+		       (l.decay_rank > 0 ? l.decay_rank : l.heads);
 	}
 }
 
@@ -130,12 +141,21 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 	ARGCHK(c.block_kind == YALM_BLOCK_SERIAL || (c.block_kind == YALM_BLOCK_PARALLEL && c.pre_norm),
 	       "yalm_seq_create: blocks are serial, or parallel with pre_norm");
 	const bool par = c.block_kind == YALM_BLOCK_PARALLEL;
-	for (int i = 0; i < c.n_layers; ++i) {
+	for (int i = 0; i < (int)L.size(); ++i) { // the n_layers entries, then their second mixers
 		const yalm_seq_layer &l = L[i];
-		const std::string at = "yalm_seq_create: layer " + std::to_string(i) + ": ";
-		ARGCHK((l.norm1 || !c.pre_norm) && (l.norm1b || par) && l.w_in && l.w_o, at + "missing tensors");
-		ARGCHK(!par || (l.ls1 && (l.ls2 || l.ff_kind == YALM_FF_NONE)), at + "a parallel block needs its scale vectors");
-		ARGCHK(l.ff_act >= YALM_ACT_DEFAULT && l.ff_act <= YALM_ACT_SILU, at + "unknown feed-forward activation");
+		const bool is_side = i >= c.n_layers;
+		const std::string at = "yalm_seq_create: " + std::string(is_side ? "second mixer " : "layer ") +
+		                       std::to_string(is_side ? i - c.n_layers : i) + ": ";
+		ARGCHK(l.w_in && l.w_o, at + "missing tensors");
+		if (is_side) {
+			ARGCHK(l.ff_kind == YALM_FF_NONE && !l.side && !l.pre_add, at + "a second mixer has no feed-forward, no vector and no side of its own");
+		} else {
+			ARGCHK((l.norm1 || !c.pre_norm) && (l.norm1b || par), at + "missing tensors");
+			ARGCHK(!l.side || (l.join_w && l.side_join_w), at + "two mixers side by side need the norm weights of their results");
+		}
+		ARGCHK(l.ff_act >= YALM_ACT_DEFAULT && l.ff_act <= YALM_ACT_RELU2 &&
+		           (l.ff_act != YALM_ACT_RELU2 || l.ff_kind == YALM_FF_PLAIN || l.ff_kind == YALM_FF_NONE),
+		       at + "unknown feed-forward activation (relu^2 belongs to the plain feed-forward)");
 		ARGCHK(!l.pre_add || i == 0 || par, at + "a vector added before an entry after the first needs parallel blocks");
 		if (latent_direct(l)) {
 			ARGCHK(l.heads > 0 && l.dim > 0 && l.vdim > 0 && l.kv_rank > 0 && l.rot_dim >= 0 && l.kv_from < 0,
@@ -181,6 +201,19 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 			}
 			ARGCHK(l.conv >= 1 && l.conv <= SEQ_MAX_TAPS, at + "convolution taps out of range");
 			ARGCHK(l.conv_w && l.a_log && l.dt_bias && l.out_norm, at + "missing delta rule tensors");
+			ARGCHK(l.decay_rank >= 0 && l.gate_rank >= 0 && (l.decay_rank == 0 || l.w_a2) && (l.gate_rank == 0 || l.w_g2) &&
+			           (l.gate_act == YALM_GATE_SILU || l.gate_act == YALM_GATE_SIGMOID),
+			       at + "bad low-rank decay / gate of the delta rule");
+		} else if (l.mixer == YALM_MIX_SSM) {
+			ARGCHK(l.heads > 0 && l.vdim > 0 && l.ssm_state > 0 && l.ssm_groups > 0 && l.heads % l.ssm_groups == 0 &&
+			           l.norm_groups > 0 && (l.heads * l.vdim) % l.norm_groups == 0,
+			       at + "bad state-space sizes");
+			if (l.ssm_state > 256) {
+				set_err(at + "a state of more than 256 rows is not implemented by the recurrence kernel");
+				return YALM_ERR_UNSUPPORTED;
+			}
+			ARGCHK(l.conv >= 1 && l.conv <= SEQ_MAX_TAPS, at + "convolution taps out of range");
+			ARGCHK(l.conv_w && l.a_log && l.dt_bias && l.d_skip && l.out_norm, at + "missing state-space tensors");
 		} else if (l.mixer == YALM_MIX_ATTN) {
 			ARGCHK(l.heads > 0 && l.kv_heads > 0 && l.heads % l.kv_heads == 0 && l.dim > 0 && l.vdim > 0,
 			       at + "bad attention sizes");
@@ -190,8 +223,12 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 			}
 			ARGCHK(l.mask_kind == YALM_MASK_CAUSAL || ((l.mask_kind == YALM_MASK_WINDOW || l.mask_kind == YALM_MASK_CHUNK) && l.mask_size > 0),
 			       at + "bad attention mask");
-			ARGCHK(l.qk_norm == YALM_QK_NONE || l.qk_norm == YALM_QK_HEAD_UNIT || (l.qk_norm == YALM_QK_WHOLE && l.q_norm && l.kv_norm),
+			ARGCHK(l.qk_norm == YALM_QK_NONE || l.qk_norm == YALM_QK_HEAD_UNIT || (l.qk_norm == YALM_QK_WHOLE && l.q_norm && l.kv_norm) ||
+			           (l.qk_norm == YALM_QK_HEAD_W && l.q_norm && l.kv_norm && l.rot_dims == 0),
 			       at + "bad query / key norm");
+			ARGCHK(l.rel_rows == 0 || (l.rel && l.rel_rows >= 2 && l.rel_max > (float)(l.rel_rows / 2)),
+			       at + "a distance bias needs its table, at least two rows and rel_max above half of them");
+			ARGCHK(l.q_temp_every >= 0, at + "bad query temperature");
 			ARGCHK(l.out_gate >= 0 && l.out_gate <= 2, at + "unknown output gate");
 			ARGCHK(l.rot_dims >= 0 && l.rot_dims <= l.dim && l.rot_dims % 2 == 0 && (l.rot_dims == 0 || l.rot_base > 0.0f),
 			       at + "rotary sizes must be even and at most dim");
@@ -209,7 +246,8 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 			           l.groups <= SEQ_MAX_GROUPS && l.experts % l.groups == 0 && l.groups_keep > 0 &&
 			           l.groups_keep <= l.groups && l.top <= l.groups_keep * (l.experts / l.groups),
 			       at + "bad router sizes");
-			ARGCHK(l.router_kind == YALM_ROUTER_SOFTMAX_TOP || (l.router_kind == YALM_ROUTER_TOP_SOFTMAX && l.groups == 1),
+			ARGCHK(l.router_kind == YALM_ROUTER_SOFTMAX_TOP || l.router_kind == YALM_ROUTER_SIGMOID_GROUPS ||
+			           (l.router_kind == YALM_ROUTER_TOP_SOFTMAX && l.groups == 1),
 			       at + "unknown router kind (the top-logits router has no groups)");
 			ARGCHK(l.router && l.w_gate && l.w_up && l.w_down && (par || ((l.norm2 || !c.pre_norm) && l.norm2b)), at + "missing expert tensors");
 			if (l.shared_ff > 0)
@@ -277,11 +315,46 @@ static int attn_setup(yalm_seq_s *q, int li) {
 	return YALM_OK;
 }
 
+// attn with a distance bias: the layer's bucketed table rel [rel_rows][heads] expanded per
+// distance, [rel_far + 1][heads], so that the kernels look a bias up by min(i - j, rel_far).
+// bucket(n) = n below half = rel_rows / 2, else min(rel_rows - 1, half + floor(ln(n / half) /
+// ln(rel_max / half) (rel_rows - half))), evaluated in double; from rel_max on every distance
+// falls into the last row.
+static int rel_setup(yalm_seq_s *q, int li) {
+	const yalm_seq_layer &l = q->L[li];
+	if (l.rel_rows <= 0)
+		return YALM_OK;
+	const int B = l.rel_rows, half = B / 2, H = l.heads;
+	const int far = std::max(half, std::min(q->c.max_tokens - 1, (int)std::ceil((double)l.rel_max)));
+	std::vector<float> rel((size_t)B * H), tab((size_t)(far + 1) * H);
+	HIPCHK(hipMemcpy(rel.data(), l.rel, rel.size() * sizeof(float), hipMemcpyDeviceToHost));
+	for (int n = 0; n <= far; ++n) {
+		int b = n;
+		if (n >= half) {
+			const double x = std::log((double)n / half) / std::log((double)l.rel_max / half) * (double)(B - half);
+			b = (int)std::min((double)(B - 1), (double)half + std::floor(x));
+		}
+		for (int h = 0; h < H; ++h)
+			tab[(size_t)n * H + h] = rel[(size_t)b * H + h];
+	}
+	q->rel_far[li] = far;
+	TRY(sallocT(q, &q->rel_dist[li], tab.size()));
+	HIPCHK(hipMemcpy(q->rel_dist[li], tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice));
+	return YALM_OK;
+}
+
 static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, yalm_stream s, Seq **out) {
 	ARGCHK(config && w && w->layers && w->embed && w->final_norm && w->head && out, "yalm_seq_create: null argument");
 	Seq *q = new Seq;
 	q->c = *config;
 	q->L.assign(w->layers, w->layers + config->n_layers);
+	q->side_of.assign(config->n_layers, -1);
+	for (int i = 0; i < config->n_layers; ++i) // second mixers follow the layers, with caches and states of their own
+		if (q->L[i].side) {
+			q->side_of[i] = (int)q->L.size();
+			q->L.push_back(*q->L[i].side);
+		}
+	q->embed_norm = w->embed_norm;
 	q->embed = w->embed;
 	q->head = w->head;
 	q->final_norm = w->final_norm;
@@ -325,9 +398,14 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 		} else if (l.mixer == YALM_MIX_ATTN) {
 			// with score mixing a portion's queries span the whole key row
 			bw = std::max({bw, (size_t)l.heads * l.dim * (l.talk ? l.kv_heads : 1), (size_t)l.heads * l.vdim});
+		} else if (l.mixer == YALM_MIX_SSM) {
+			const size_t cc = (size_t)l.heads * l.vdim + 2 * (size_t)l.ssm_groups * l.ssm_state;
+			bw = std::max({bw, cc, (size_t)2 * l.heads});
+			arena += (size_t)l.heads * l.ssm_state * l.vdim + (size_t)(l.conv - 1) * cc;
 		} else {
 			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
-			bw = std::max({bw, cc, (size_t)l.heads * l.vdim, (size_t)2 * l.heads});
+			// beta and per-head decay, then (decay_rank) one decay per head and key channel
+			bw = std::max({bw, cc, (size_t)l.heads * l.vdim, (size_t)2 * l.heads + (l.decay_rank > 0 ? (size_t)l.heads * l.dim : 0)});
 			arena += (size_t)l.heads * l.dim * l.vdim + (size_t)(l.conv - 1) * cc;
 		}
 		if (l.ff_kind == YALM_FF_DENSE || l.ff_kind == YALM_FF_PLAIN)
@@ -347,6 +425,18 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	STRY(sallocT(q, &q->Y, cap * c.width));
 	if (c.block_kind == YALM_BLOCK_PARALLEL)
 		STRY(sallocT(q, &q->Y2, cap * c.width));
+	q->Yout = q->Y;
+	{
+		bool own_ff_norm = false, sides = false;
+		for (int i = 0; i < c.n_layers; ++i) {
+			own_ff_norm |= c.block_kind == YALM_BLOCK_PARALLEL && q->L[i].norm2 && q->L[i].ff_kind != YALM_FF_NONE;
+			sides |= q->side_of[i] >= 0;
+		}
+		if (own_ff_norm)
+			STRY(sallocT(q, &q->Hn2, cap * c.width));
+		if (sides)
+			STRY(sallocT(q, &q->Y3, cap * c.width));
+	}
 	STRY(sallocT(q, &q->Z, cap * zw));
 	for (int i = 0; i < 4; ++i)
 		STRY(sallocT(q, &q->B[i], cap * bw));
@@ -370,8 +460,8 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 		q->att_splits = std::max(1, std::min(32, cdiv(c.max_tokens, 2 * ATT_KT)));
 		size_t part = (size_t)(4 * ATT_BR + GEMV_MAX_M * max_h) * q->att_splits * (att_rank4(max_rank) + 4);
 		// attn: the keys a single token can see, split so that a workgroup walks one tile (up to 64 splits)
-		q->attn_splits.assign(c.n_layers, 1);
-		for (int i = 0; i < c.n_layers; ++i) {
+		q->attn_splits.assign(q->L.size(), 1);
+		for (int i = 0; i < (int)q->L.size(); ++i) {
 			const yalm_seq_layer &l = q->L[i];
 			if (l.mixer != YALM_MIX_ATTN && !latent_direct(l))
 				continue;
@@ -402,14 +492,17 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	}
 	q->arena_floats = arena;
 	STRY(sallocT(q, &q->arena, arena));
-	q->cache.assign(c.n_layers, nullptr);
-	q->S.assign(c.n_layers, nullptr);
-	q->conv.assign(c.n_layers, nullptr);
-	q->vcache.assign(c.n_layers, nullptr);
-	q->rot_freq.assign(c.n_layers, nullptr);
-	q->rot_mag.assign(c.n_layers, 1.0f);
+	const int NL = (int)q->L.size();
+	q->cache.assign(NL, nullptr);
+	q->S.assign(NL, nullptr);
+	q->conv.assign(NL, nullptr);
+	q->vcache.assign(NL, nullptr);
+	q->rot_freq.assign(NL, nullptr);
+	q->rot_mag.assign(NL, 1.0f);
+	q->rel_dist.assign(NL, nullptr);
+	q->rel_far.assign(NL, 0);
 	size_t off = 0;
-	for (int i = 0; i < c.n_layers; ++i) {
+	for (int i = 0; i < NL; ++i) {
 		const yalm_seq_layer &l = q->L[i];
 		if (latent_direct(l)) {
 			STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * (l.kv_rank + l.rot_dim) * (bf ? 2 : 4)));
@@ -423,11 +516,18 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 			STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * l.kv_heads * l.dim * (bf ? 2 : 4)));
 			STRY(salloc(q, &q->vcache[i], (size_t)c.max_tokens * l.kv_heads * l.vdim * (bf ? 2 : 4)));
 			STRY(attn_setup(q, i));
+			STRY(rel_setup(q, i));
 		} else if (l.mixer == YALM_MIX_RGLRU) {
 			q->S[i] = q->arena + off;
 			off += l.rec_width;
 			q->conv[i] = q->arena + off;
 			off += (size_t)(l.conv - 1) * l.rec_width;
+		} else if (l.mixer == YALM_MIX_SSM) {
+			const size_t cc = (size_t)l.heads * l.vdim + 2 * (size_t)l.ssm_groups * l.ssm_state;
+			q->S[i] = q->arena + off;
+			off += (size_t)l.heads * l.ssm_state * l.vdim;
+			q->conv[i] = q->arena + off;
+			off += (size_t)(l.conv - 1) * cc;
 		} else {
 			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
 			q->S[i] = q->arena + off;
@@ -532,7 +632,8 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 	// output columns past the last multiple of 128 (a few gate rows closing an input projection)
 	// run on the general kernel as a second, narrow product
 	const bool pair = a.W2 != nullptr && (a.epi == EPI_GLU_GELU || a.epi == EPI_GLU_CLAMP || a.epi == EPI_GLU_SILU) && !a.bias;
-	const bool single = !a.W2 && (a.epi == EPI_NONE || a.epi == EPI_GELU);
+	const bool single = !a.W2 && (a.epi == EPI_NONE || a.epi == EPI_GELU || a.epi == EPI_RELU2);
+	const int act1 = a.epi == EPI_GELU ? 1 : (a.epi == EPI_RELU2 ? 2 : 0); // the large-tile door's activation
 	const int n_big = pair ? (a.N % 64 == 0 ? a.N : 0) : (single ? a.N & ~127 : 0);
 	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.rows && !a.w_sel && a.z_split == 0 && a.ldw == a.K &&
 	    a.K % 64 == 0 && n_big > 0 && (a.N - n_big <= 64 || (!pair && a.N - n_big < 128))) {
@@ -544,13 +645,13 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 		    pair ? pf_gemm_glu_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, (const uint16_t *)a.W2, a.N, a.C, a.ldc,
 		                            a.epi == EPI_GLU_GELU ? 1 : (a.epi == EPI_GLU_CLAMP ? 2 : 3), a.limit, q->stream)
 		         : pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, n_big, a.C, a.ldc, a.bias,
-		                        a.epi == EPI_GELU ? 1 : 0, q->stream);
+		                        act1, q->stream);
 		if (rc == YALM_OK && !pair && n_big < a.N && a.N >= 128) {
 			// the last 128 columns as one more large tile: it computes the columns below n_big a
 			// second time (the same kernel on the same operands: the same values) and the tail
 			const int c0 = a.N - 128;
 			const int rc2 = pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W + (size_t)c0 * a.ldw, 128, a.C + c0,
-			                             a.ldc, a.bias ? a.bias + c0 : nullptr, a.epi == EPI_GELU ? 1 : 0, q->stream);
+			                             a.ldc, a.bias ? a.bias + c0 : nullptr, act1, q->stream);
 			if (rc2 != YALM_ERR_UNSUPPORTED)
 				return rc2;
 		}
@@ -650,7 +751,7 @@ static int mixer_latent(Seq *q, int li, int n) {
 		a.c_bs = V;
 		TRY(gemm(q, a, H));
 	}
-	return gemm(q, plain(qh, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V));
+	return gemm(q, plain(qh, H * V, l.w_o, H * V, q->Yout, c.width, n, c.width, H * V));
 }
 
 static int conv_launch(Seq *q, const float *Z, int ldz, int col0, int C, int taps, const float *w, const float *bias,
@@ -702,7 +803,34 @@ static int mixer_rglru(Seq *q, int li, int n) {
 		seq_rglru_walk_kernel<<<cdiv(W, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->S[li], so, n);
 	}
 	HIPCHK(hipGetLastError());
-	return gemm(q, plain(so, W, l.w_o, W, q->Y, c.width, n, c.width, W));
+	return gemm(q, plain(so, W, l.w_o, W, q->Yout, c.width, n, c.width, W));
+}
+
+// The recurrence kernel over a portion: the gated delta rule (ssm = false; gv: one decay per head
+// and key channel) or the state-space walk (ssm = true). K: key / state size, P: value size.
+static int delta_launch(Seq *q, const float *qkv, int ldq, int qo, int ko, int vo, int KH, int K, int H, int P,
+                        const float *bg, const float *gv, const float *dskip, float *state, float *o, int n, bool ssm) {
+	const dim3 g(cdiv(P, SEQ_THREADS / 8), H);
+	const int R = cdiv(K, 8);
+#define DELTA_LAUNCH(RR, TC)                                                                                           \
+	do {                                                                                                               \
+		if (ssm)                                                                                                       \
+			seq_delta_kernel<RR, TC, true, false><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, ldq, qo, ko, vo, KH, K, H, P, bg, \
+			                                                                        nullptr, dskip, state, o, n);          \
+		else if (gv)                                                                                                   \
+			seq_delta_kernel<RR, TC, false, true><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, ldq, qo, ko, vo, KH, K, H, P, bg, \
+			                                                                        gv, nullptr, state, o, n);             \
+		else                                                                                                           \
+			seq_delta_kernel<RR, TC, false, false><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, ldq, qo, ko, vo, KH, K, H, P,   \
+			                                                                         bg, nullptr, nullptr, state, o, n);   \
+	} while (0)
+	if (R <= 4) DELTA_LAUNCH(4, 16);
+	else if (R <= 8) DELTA_LAUNCH(8, 16);
+	else if (R <= 16) DELTA_LAUNCH(16, 16);
+	else DELTA_LAUNCH(32, 8);
+#undef DELTA_LAUNCH
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
 }
 
 static int mixer_delta(Seq *q, int li, int n) {
@@ -710,24 +838,52 @@ static int mixer_delta(Seq *q, int li, int n) {
 	const yalm_seq_config &c = q->c;
 	const int H = l.heads, KH = l.kv_heads, D = l.dim, V = l.vdim;
 	const int CQ = KH * D, CV = H * V, cc = 2 * CQ + CV, zin = in_rows(l);
-	const int gcol = cc, bcol = cc + CV, acol = bcol + H;
+	const int gcol = cc, bcol = cc + (l.gate_rank > 0 ? l.gate_rank : CV), acol = bcol + H;
 	float *qkv = q->B[0], *bg = q->B[1], *o = q->B[2], *on = q->B[3];
+	// one decay per head and key channel: its inputs, then the decays, follow the [n][2 H] factors
+	float *gv = l.decay_rank > 0 ? bg + (size_t)n * 2 * H : nullptr;
 	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
 	TRY(conv_launch(q, q->Z, zin, 0, cc, l.conv, l.conv_w, nullptr, 1, q->conv[li], qkv, n));
+	if (gv) // the low-rank decay's second factor
+		TRY(gemm(q, plain(q->Z + acol, zin, l.w_a2, l.decay_rank, gv, H * D, n, H * D, l.decay_rank)));
 	seq_delta_prep_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, q->Z, zin, bcol, acol, H, l.a_log, l.dt_bias,
-	                                                        bg);
-	const dim3 g(cdiv(V, SEQ_THREADS / 8), H);
-	const int R = cdiv(D, 8);
-#define DELTA_LAUNCH(RR, TC)                                                                                           \
-	seq_delta_kernel<RR, TC><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, H, V, bg, q->S[li], o, n)
-	if (R <= 4) DELTA_LAUNCH(4, 16);
-	else if (R <= 8) DELTA_LAUNCH(8, 16);
-	else if (R <= 16) DELTA_LAUNCH(16, 16);
-	else DELTA_LAUNCH(32, 8);
-#undef DELTA_LAUNCH
-	seq_delta_out_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(o, H, V, l.out_norm, c.norm_eps, q->Z, zin, gcol, on);
+	                                                        bg, gv);
 	HIPCHK(hipGetLastError());
-	return gemm(q, plain(on, CV, l.w_o, CV, q->Y, c.width, n, c.width, CV));
+	const float *gl = q->Z;
+	int ldg = zin, gc = gcol;
+	if (l.gate_rank > 0) { // the low-rank gate's second factor; the gated read-out then overwrites its logits
+		TRY(gemm(q, plain(q->Z + gcol, zin, l.w_g2, l.gate_rank, on, CV, n, CV, l.gate_rank)));
+		gl = on;
+		ldg = CV;
+		gc = 0;
+	}
+	TRY(delta_launch(q, qkv, cc, 0, CQ, 2 * CQ, KH, D, H, V, bg, gv, nullptr, q->S[li], o, n, false));
+	seq_delta_out_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(o, H, V, l.out_norm, c.norm_eps, gl, ldg, gc, on,
+	                                                       l.gate_act == YALM_GATE_SIGMOID);
+	HIPCHK(hipGetLastError());
+	return gemm(q, plain(on, CV, l.w_o, CV, q->Yout, c.width, n, c.width, CV));
+}
+
+// Selective state-space layer: one input projection (gate | x | B | C | step), the convolution
+// with silu over x | B | C, per-head step sizes and decays, the recurrence (the delta rule's
+// kernel in its state-space form: B as keys, C as queries, x as values), the gated result
+// rms-normed in equal parts, the output projection.
+static int mixer_ssm(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const int H = l.heads, P = l.vdim, N = l.ssm_state, G = l.ssm_groups;
+	const int inner = H * P, GN = G * N, cc = inner + 2 * GN, zin = in_rows(l);
+	float *xbc = q->B[0], *bg = q->B[1], *y = q->B[2], *yn = q->B[3];
+	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
+	TRY(conv_launch(q, q->Z, zin, inner, cc, l.conv, l.conv_w, l.conv_b, 1, q->conv[li], xbc, n));
+	seq_ssm_prep_kernel<<<cdiv(n * H, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(q->Z, zin, inner + cc, H, l.a_log,
+	                                                                            l.dt_bias, bg, n);
+	HIPCHK(hipGetLastError());
+	TRY(delta_launch(q, xbc, cc, inner + GN, inner, 0, G, N, H, P, bg, nullptr, l.d_skip, q->S[li], y, n, true));
+	seq_gated_part_norm_kernel<<<dim3(n, l.norm_groups), SEQ_THREADS, 0, q->stream>>>(y, inner, l.norm_groups, q->Z, zin, 0,
+	                                                                                  l.out_norm, c.norm_eps, yn);
+	HIPCHK(hipGetLastError());
+	return gemm(q, plain(yn, inner, l.w_o, inner, q->Yout, c.width, n, c.width, inner));
 }
 
 // ---- the closing norm of a single token, owed to the product that reads the stream next
@@ -937,6 +1093,10 @@ static int mixer_attn(Seq *q, int li, int n) {
 	a.k_w = l.kv_norm;
 	a.temp = l.head_temp;
 	a.talk = l.talk;
+	a.rel_dist = q->rel_dist[li];
+	a.rel_far = q->rel_far[li];
+	a.q_temp_coef = l.q_temp_coef;
+	a.q_temp_every = l.q_temp_every;
 	a.eps = c.norm_eps;
 	// portions: the projection kernel (one workgroup per token) mixes the queries itself
 	a.q_mixed = l.talk && n > GEMV_MAX_M ? 1 : 0;
@@ -958,7 +1118,7 @@ static int mixer_attn(Seq *q, int li, int n) {
 	const float *ge = l.out_gate == 2 ? q->Z + (zin - H * V) : nullptr; // elementwise gate logits close the Z rows
 	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, Q, gp, ctx, nullptr, nullptr, ge, zin)
 	       : attn_core_t<float>(q, li, n, a, Q, gp, ctx, nullptr, nullptr, ge, zin));
-	GemmArgs o = plain(ctx, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V);
+	GemmArgs o = plain(ctx, H * V, l.w_o, H * V, q->Yout, c.width, n, c.width, H * V);
 	o.bias = l.o_bias;
 	return gemm(q, o);
 }
@@ -1075,7 +1235,7 @@ static int mixer_latent_direct(Seq *q, int li, int n) {
 			TRY(gemm(q, b, H));
 		}
 	}
-	GemmArgs o = plain(oh, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V);
+	GemmArgs o = plain(oh, H * V, l.w_o, H * V, q->Yout, c.width, n, c.width, H * V);
 	o.bias = l.o_bias;
 	return gemm(q, o);
 }
@@ -1085,7 +1245,7 @@ static int ff_plain(Seq *q, int li, int n, float *out) {
 	const yalm_seq_layer &l = q->L[li];
 	const yalm_seq_config &c = q->c;
 	GemmArgs a = plain(q->In, c.width, l.w_up, c.width, q->B[0], l.ff, n, l.ff, c.width);
-	a.epi = EPI_GELU;
+	a.epi = l.ff_act == YALM_ACT_RELU2 ? EPI_RELU2 : EPI_GELU;
 	TRY(gemm_in(q, a));
 	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, out, c.width, n, c.width, l.ff));
 }
@@ -1116,7 +1276,7 @@ static int ff_moe(Seq *q, int li, int n) {
 	const yalm_seq_config &c = q->c;
 	const int E = l.experts, top = l.top, ff = l.ff, slots = n * top;
 	float *hx = q->B[0], *yx = q->B[1], *hs = q->B[2], *ys = q->B[3];
-	seq_router_kernel<<<n, SEQ_THREADS, (E + l.groups) * sizeof(float), q->stream>>>(q->In, c.width, l.router, E, top, l.groups,
+	seq_router_kernel<<<n, SEQ_THREADS, (2 * E + l.groups) * sizeof(float), q->stream>>>(q->In, c.width, l.router, E, top, l.groups,
 	                                                                    l.groups_keep, l.router_scale,
 	                                                                    l.shared_ff > 0 ? l.shared_sg : nullptr, q->idx,
 	                                                                    q->wt, q->sgate, l.router_kind, l.router_bias);
@@ -1184,7 +1344,8 @@ static int par_close(Seq *q, int li, int n) {
 #define PC_ARGS                                                                                                        \
 	q->X, q->Y, l.ls1, (l.ff_kind != YALM_FF_NONE && !moe) ? q->Y2 : nullptr, l.ls2, moe ? q->B[1] : nullptr, q->wt,    \
 	    moe ? l.top : 0, moe && l.shared_ff > 0 ? q->B[3] : nullptr, gated ? q->sgate : nullptr, dump,                 \
-	    nx ? nx->pre_add : nullptr, c.norm_eps, c.width, nx ? nx->norm1 : nullptr, q->Hn, (int)q->ln
+	    nx ? nx->pre_add : nullptr, c.norm_eps, c.width, nx ? nx->norm1 : nullptr, q->Hn, (int)q->ln,                  \
+	    (nx && nx->ff_kind != YALM_FF_NONE) ? nx->norm2 : nullptr, q->Hn2
 	if (c.width <= 4 * SEQ_THREADS)
 		seq_par_close_reg_kernel<4><<<n, SEQ_THREADS, 0, q->stream>>>(PC_ARGS);
 	else if (c.width <= 8 * SEQ_THREADS)
@@ -1224,6 +1385,9 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	const yalm_seq_config &c = q->c;
 	const bool pre = c.pre_norm != 0; // else the sublayers read the stream itself and no opening norm is computed
 	const float *first_norm = pre ? q->L[0].norm1 : nullptr;
+	const bool par = c.block_kind == YALM_BLOCK_PARALLEL;
+	// a parallel block whose feed-forward has a norm of its own reads Hn2 = norm2(x)
+	const float *first_norm2 = (par && q->L[0].ff_kind != YALM_FF_NONE) ? q->L[0].norm2 : nullptr;
 	if (!pre) { // every portion starts in the same row of the stream (the greedy graph's pointers are static)
 		q->X = q->Xbase;
 		q->In = q->X;
@@ -1241,35 +1405,58 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	if (c.weight_dtype == YALM_F32)
 		seq_embed_kernel<WF32><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
 		                                                         c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
-		                                                         q->Hn, (int)q->ln, q->L[0].pre_add);
+		                                                         q->Hn, (int)q->ln, q->L[0].pre_add, q->embed_norm, first_norm2,
+		                                                         q->Hn2);
 	else
 		seq_embed_kernel<WBF16><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
 		                                                          c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
-		                                                          q->Hn, (int)q->ln, q->L[0].pre_add);
+		                                                          q->Hn, (int)q->ln, q->L[0].pre_add, q->embed_norm, first_norm2,
+		                                                          q->Hn2);
 	HIPCHK(hipGetLastError());
-	const bool par = c.block_kind == YALM_BLOCK_PARALLEL;
+	auto run_mixer = [&](int mi) {
+		const yalm_seq_layer &m = q->L[mi];
+		if (latent_direct(m))
+			return mixer_latent_direct(q, mi, n);
+		if (m.mixer == YALM_MIX_LATENT)
+			return mixer_latent(q, mi, n);
+		if (m.mixer == YALM_MIX_RGLRU)
+			return mixer_rglru(q, mi, n);
+		if (m.mixer == YALM_MIX_ATTN)
+			return mixer_attn(q, mi, n);
+		if (m.mixer == YALM_MIX_SSM)
+			return mixer_ssm(q, mi, n);
+		return mixer_delta(q, mi, n);
+	};
 	for (int li = 0; li < c.n_layers; ++li) {
 		const yalm_seq_layer &l = q->L[li];
 		const float *next = pre && li + 1 < c.n_layers ? q->L[li + 1].norm1 : nullptr;
-		if (l.mixer != YALM_MIX_ATTN)
-			TRY(flush_norm(q, n)); // only the attention mixer's input projection takes an owed norm
-		if (latent_direct(l))
-			TRY(mixer_latent_direct(q, li, n));
-		else if (l.mixer == YALM_MIX_LATENT)
-			TRY(mixer_latent(q, li, n));
-		else if (l.mixer == YALM_MIX_RGLRU)
-			TRY(mixer_rglru(q, li, n));
-		else if (l.mixer == YALM_MIX_ATTN)
-			TRY(mixer_attn(q, li, n));
-		else
-			TRY(mixer_delta(q, li, n));
-		if (par) { // both sublayers read Hn; the feed-forward's result goes beside the mixer's
+		const int side = q->side_of[li];
+		if (l.mixer != YALM_MIX_ATTN || side >= 0)
+			TRY(flush_norm(q, n)); // only a lone attention mixer's input projection takes an owed norm
+		q->Yout = q->Y;
+		TRY(run_mixer(li));
+		if (side >= 0) { // the second mixer reads the same input; the two normed results are summed into Y
+			q->Yout = q->Y3;
+			const int rc = run_mixer(side);
+			q->Yout = q->Y;
+			TRY(rc);
+			seq_pair_join_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(q->Y, q->Y3, l.join_w, l.side_join_w, l.join_scale,
+			                                                       c.norm_eps, c.width);
+			HIPCHK(hipGetLastError());
+		}
+		if (par) { // both sublayers read norms of the same stream; the feed-forward's result goes beside the mixer's
+			const float *mix_in = q->In;
+			if (l.norm2 && l.ff_kind != YALM_FF_NONE)
+				q->In = q->Hn2;
+			int rc = YALM_OK;
 			if (l.ff_kind == YALM_FF_DENSE)
-				TRY(ff_dense(q, li, n, q->Y2));
+				rc = ff_dense(q, li, n, q->Y2);
 			else if (l.ff_kind == YALM_FF_PLAIN)
-				TRY(ff_plain(q, li, n, q->Y2));
+				rc = ff_plain(q, li, n, q->Y2);
 			else if (l.ff_kind == YALM_FF_MOE)
-				TRY(ff_moe(q, li, n));
+				rc = ff_moe(q, li, n);
+			q->In = mix_in;
+			TRY(rc);
 			TRY(par_close(q, li, n));
 			continue;
 		}

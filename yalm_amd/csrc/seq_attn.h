@@ -36,7 +36,19 @@ struct AttnArgs {
 	int q_mixed;              // talk: the projection kernel has already written the mixed queries [t][H][G D]
 	int KL = 0, VL = 0;       // entries per key / value cache row (head g's keys at column g D, values at g V)
 	const float *sink_w = nullptr; // sink: [H] scores of the valueless key, unscaled; null: 0
+	// a learned bias per head and distance, added to the scaled score: rel_dist[min(i - j, rel_far)][h]
+	// (the bucketed table of the layer expanded per distance at creation), or null
+	const float *rel_dist = nullptr;
+	int rel_far = 0;
+	// q_temp_every > 0: the query at position p times 1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1)
+	float q_temp_coef = 0.0f;
+	int q_temp_every = 0;
 };
+
+// The bias of head h's score between a query and a key `dist` positions before it.
+__device__ __forceinline__ float attn_rel_bias(const AttnArgs &a, int h, int dist) {
+	return a.rel_dist ? a.rel_dist[(size_t)min(max(dist, 0), a.rel_far) * a.H + h] : 0.0f;
+}
 
 // The softmax's starting state for head h: with a sink, a valueless key of score sink_w[h] (or 0)
 // has already been seen (running maximum = its score, running sum 1).
@@ -201,16 +213,21 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 		}
 		ss = wave_sum(ss);
 		float mul = 1.0f;
-		if (kind == 2 ? a.v_norm != 0 : a.qk_norm == YALM_QK_HEAD_UNIT)
+		const bool head_w = kind < 2 && a.qk_norm == YALM_QK_HEAD_W;
+		if (kind == 2 ? a.v_norm != 0 : (a.qk_norm == YALM_QK_HEAD_UNIT || head_w))
 			mul = 1.0f / sqrtf(ss / (float)n + a.eps);
-		if (kind == 0)
+		if (kind == 0) {
 			mul *= a.scale * (a.temp ? a.temp[hh] : 1.0f);
+			if (a.q_temp_every > 0)
+				mul *= 1.0f + a.q_temp_coef * logf((float)((p + 1) / a.q_temp_every) + 1.0f);
+		}
+		const float *hw = head_w ? (kind == 0 ? a.q_w : a.k_w) : nullptr;
 #pragma unroll
 		for (int e = 0; e < 4; ++e) {
 			const int d = lane + 64 * e;
 			if (d >= n)
 				continue;
-			const float v = val[e] * mul;
+			const float v = val[e] * mul * (hw ? hw[d] : 1.0f);
 			if (kind == 0) {
 				if (a.q_mixed)
 					qsh[hh * a.D + d] = v;
@@ -517,7 +534,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 		for (int r = wave; r < R; r += SEQ_THREADS / 64) {
 			const int j = kt + lane;
 			const bool vis = j >= rlo[r] && j <= rhi[r] && j < k_end;
-			const float sv = vis ? ps[r * SA_KT + lane] : -FLT_MAX;
+			const float sv = vis ? ps[r * SA_KT + lane] + attn_rel_bias(a, h0 + r % Hb, rhi[r] - j) : -FLT_MAX;
 			const float mold = mrun[r], lold = lrun[r];
 			const float mnew = fmaxf(mold, wave_max(sv));
 			const float p = vis ? expf(sv - mnew) : 0.0f;
@@ -746,7 +763,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const floa
 #pragma unroll
 			for (int w = 0; w < NW; ++w)
 				sv += pw[(w * Hb + r) * SA_KT + lane];
-			sv = live ? sv : -FLT_MAX;
+			sv = live ? sv + attn_rel_bias(a, h0 + r, pos - j) : -FLT_MAX;
 			const float mold = mrun[r], lold = lrun[r];
 			const float mnew = fmaxf(mold, wave_max(sv));
 			const float p = live ? expf(sv - mnew) : 0.0f;
@@ -1013,7 +1030,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 			for (int r = 0; r < 4; ++r) {
 				const int j0 = kt + lr, j1 = kt + 16 + lr;
 				const bool v0 = j0 >= lo_[r] && j0 <= hi_[r], v1 = j1 >= lo_[r] && j1 <= hi_[r];
-				const float s0 = v0 ? sacc[0][r] : -FLT_MAX, s1 = v1 ? sacc[1][r] : -FLT_MAX;
+				const float s0 = v0 ? sacc[0][r] + attn_rel_bias(a, h, hi_[r] - j0) : -FLT_MAX;
+				const float s1 = v1 ? sacc[1][r] + attn_rel_bias(a, h, hi_[r] - j1) : -FLT_MAX;
 				const float mnew = fmaxf(mrun[r], row16_max(fmaxf(s0, s1)));
 				const float p0 = v0 ? expf(s0 - mnew) : 0.0f, p1 = v1 ? expf(s1 - mnew) : 0.0f;
 				al[r] = expf(mrun[r] - mnew);

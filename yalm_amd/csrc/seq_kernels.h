@@ -65,9 +65,11 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 
 // ------------------------------------------------------------------ embedding
 // X[t] = embed[token] * scale (+ the interleaved (sin, cos) position vector of position
-// st->pos + t if inv_freq) (+ pre_add, a vector the first layer adds to the stream before its
+// st->pos + t if inv_freq), rms-normed with weight e_norm if e_norm (no mean taken off)
+// (+ pre_add, a vector the first layer adds to the stream before its
 // opening norm); tokens == nullptr: the single device-resident token of the greedy
-// loop. w_next != nullptr: also Hn[t] = norm(X[t]) * w_next, the first layer's opening norm.
+// loop. w_next != nullptr: also Hn[t] = norm(X[t]) * w_next, the first layer's opening norm,
+// and with w_next2 Hn2[t] = norm(X[t]) * w_next2 (the norm its feed-forward reads).
 template <class WT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState *__restrict__ st,
                                                                 const int *__restrict__ tokens,
@@ -76,7 +78,10 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
                                                                 int vocab, float scale, float *__restrict__ X,
                                                                 const float *__restrict__ w_next, float eps,
                                                                 float *__restrict__ Hn, int ln,
-                                                                const float *__restrict__ pre_add = nullptr) {
+                                                                const float *__restrict__ pre_add = nullptr,
+                                                                const float *__restrict__ e_norm = nullptr,
+                                                                const float *__restrict__ w_next2 = nullptr,
+                                                                float *__restrict__ Hn2 = nullptr) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	int tok = tokens ? tokens[t] : st->token;
@@ -90,11 +95,24 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
 			pe = (i & 1) ? cosf(ang) : sinf(ang);
 		}
 		float v = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
-		if (pre_add)
+		if (pre_add && !e_norm)
 			v += pre_add[i];
 		X[(size_t)t * width + i] = v;
 		ss = fmaf(v, v, ss);
 		sm += v;
+	}
+	if (e_norm) { // the embedding's own norm (each thread re-reads its own entries)
+		const float r0 = 1.0f / sqrtf(block_sum(ss, red) / (float)width + eps);
+		ss = 0.0f;
+		sm = 0.0f;
+		for (int i = threadIdx.x; i < width; i += SEQ_THREADS) {
+			float v = X[(size_t)t * width + i] * r0 * e_norm[i];
+			if (pre_add)
+				v += pre_add[i];
+			X[(size_t)t * width + i] = v;
+			ss = fmaf(v, v, ss);
+			sm += v;
+		}
 	}
 	if (!w_next)
 		return;
@@ -110,8 +128,12 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
 	}
 	ss = block_sum(ss, red);
 	const float r = 1.0f / sqrtf(ss / (float)width + eps);
-	for (int i = threadIdx.x; i < width; i += SEQ_THREADS)
-		Hn[(size_t)t * width + i] = (X[(size_t)t * width + i] - mu) * r * w_next[i];
+	for (int i = threadIdx.x; i < width; i += SEQ_THREADS) {
+		const float v = (X[(size_t)t * width + i] - mu) * r;
+		Hn[(size_t)t * width + i] = v * w_next[i];
+		if (w_next2)
+			Hn2[(size_t)t * width + i] = v * w_next2[i];
+	}
 }
 
 // ------------------------------------------------------------------ norms
@@ -329,7 +351,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__rest
 // Ys[t], the shared expert; sgate == nullptr: + Ys[t]), summed in slot order. dump != nullptr:
 // the row after the sums is also written there (the stream as the block leaves it). Then
 // X[t] += add (the vector the next layer adds before its opening norm) and, if w_next, Hn[t]
-// = norm(X[t]) * w_next. Dynamic LDS: n floats.
+// = norm(X[t]) * w_next and, with w_next2, Hn2[t] = norm(X[t]) * w_next2 (the norm the next
+// block's feed-forward reads). s1 / s2 == nullptr: scale 1. Dynamic LDS: n floats.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__restrict__ X, const float *__restrict__ Y1,
                                                                     const float *__restrict__ s1,
                                                                     const float *__restrict__ Y2,
@@ -341,23 +364,25 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__res
                                                                     float *__restrict__ dump,
                                                                     const float *__restrict__ add, float eps, int n,
                                                                     const float *__restrict__ w_next,
-                                                                    float *__restrict__ Hn, int ln) {
+                                                                    float *__restrict__ Hn, int ln,
+                                                                    const float *__restrict__ w_next2 = nullptr,
+                                                                    float *__restrict__ Hn2 = nullptr) {
 	extern __shared__ float row[];
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	float *x = X + (size_t)t * n;
 	float ss = 0.0f, sm = 0.0f;
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
-		float v = fmaf(s1[i], Y1[(size_t)t * n + i], x[i]);
+		float v = fmaf(s1 ? s1[i] : 1.0f, Y1[(size_t)t * n + i], x[i]);
 		if (Yx) {
 			float f = 0.0f;
 			for (int k = 0; k < top; ++k)
 				f = fmaf(wt[(size_t)t * top + k], Yx[((size_t)t * top + k) * n + i], f);
 			if (Ys)
 				f = fmaf(sgate ? sgate[t] : 1.0f, Ys[(size_t)t * n + i], f);
-			v = fmaf(s2[i], f, v);
+			v = fmaf(s2 ? s2[i] : 1.0f, f, v);
 		} else if (Y2) {
-			v = fmaf(s2[i], Y2[(size_t)t * n + i], v);
+			v = fmaf(s2 ? s2[i] : 1.0f, Y2[(size_t)t * n + i], v);
 		}
 		if (dump)
 			dump[(size_t)t * n + i] = v;
@@ -381,8 +406,12 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__res
 	}
 	ss = block_sum(ss, red);
 	const float r = 1.0f / sqrtf(ss / (float)n + eps);
-	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
-		Hn[(size_t)t * n + i] = (row[i] - mu) * r * w_next[i];
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		const float v = (row[i] - mu) * r;
+		Hn[(size_t)t * n + i] = v * w_next[i];
+		if (w_next2)
+			Hn2[(size_t)t * n + i] = v * w_next2[i];
+	}
 }
 
 // The same seam with the row in registers (rows of up to E * SEQ_THREADS entries): every
@@ -399,7 +428,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_reg_kernel(float *_
                                                                         float *__restrict__ dump,
                                                                         const float *__restrict__ add, float eps, int n,
                                                                         const float *__restrict__ w_next,
-                                                                        float *__restrict__ Hn, int ln) {
+                                                                        float *__restrict__ Hn, int ln,
+                                                                        const float *__restrict__ w_next2 = nullptr,
+                                                                        float *__restrict__ Hn2 = nullptr) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	float x[E], y1[E], a1[E], f[E], a2[E], ad[E], wn[E];
@@ -410,8 +441,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_reg_kernel(float *_
 		const bool in = i < n;
 		x[e] = in ? X[(size_t)t * n + i] : 0.0f;
 		y1[e] = in ? Y1[(size_t)t * n + i] : 0.0f;
-		a1[e] = in ? s1[i] : 0.0f;
-		a2[e] = (in && ff) ? s2[i] : 0.0f;
+		a1[e] = in ? (s1 ? s1[i] : 1.0f) : 0.0f;
+		a2[e] = (in && ff) ? (s2 ? s2[i] : 1.0f) : 0.0f;
 		ad[e] = (in && add) ? add[i] : 0.0f;
 		wn[e] = (in && w_next) ? w_next[i] : 0.0f;
 		f[e] = (in && Y2 && !Yx) ? Y2[(size_t)t * n + i] : 0.0f;
@@ -468,9 +499,33 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_reg_kernel(float *_
 #pragma unroll
 	for (int e = 0; e < E; ++e) {
 		const int i = threadIdx.x + e * SEQ_THREADS;
-		if (i < n)
+		if (i < n) {
 			Hn[(size_t)t * n + i] = x[e] * r * wn[e];
+			if (w_next2)
+				Hn2[(size_t)t * n + i] = x[e] * r * w_next2[i];
+		}
 	}
+}
+
+// Two mixers side by side: Ya[t] <- scale (rms(Ya[t]) wa + rms(Yb[t]) wb), each row divided by
+// its own root mean square over n (no mean taken off). One workgroup per token.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_pair_join_kernel(float *__restrict__ Ya, const float *__restrict__ Yb,
+                                                                    const float *__restrict__ wa,
+                                                                    const float *__restrict__ wb, float scale, float eps,
+                                                                    int n) {
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x;
+	float *a = Ya + (size_t)t * n;
+	const float *b = Yb + (size_t)t * n;
+	float sa = 0.0f, sb = 0.0f;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		sa = fmaf(a[i], a[i], sa);
+		sb = fmaf(b[i], b[i], sb);
+	}
+	const float ra = scale / sqrtf(block_sum(sa, red) / (float)n + eps);
+	const float rb = scale / sqrtf(block_sum(sb, red) / (float)n + eps);
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
+		a[i] = a[i] * ra * wa[i] + b[i] * rb * wb[i];
 }
 
 // C[t][j] *= sigmoid(Z[t][col0 + j]), j < n: an elementwise output gate whose logits are
@@ -485,7 +540,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_gate_mul_kernel(float *__rest
 }
 
 // ------------------------------------------------------------------ matrix products
-enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3, EPI_GELU = 4, EPI_GLU_SILU = 5 };
+enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3, EPI_GELU = 4, EPI_GLU_SILU = 5, EPI_RELU2 = 6 };
 
 // C[c_row(m)][n] = epi(sum_k A[a_row(m)][k] W[n][k]) for every batch z = blockIdx.z.
 struct GemmArgs {
@@ -529,6 +584,10 @@ __device__ __forceinline__ float epi_apply(const GemmArgs &a, float v, float v2,
 	case EPI_GLU_SILU: return sq_silu(v) * v2;
 	case EPI_SIGMOID: return sq_sigmoid(v + b);
 	case EPI_GELU: return sq_gelu_tanh(v + b);
+	case EPI_RELU2: {
+		const float r = fmaxf(v + b, 0.0f);
+		return r * r;
+	}
 	default: return v + b;
 	}
 }
@@ -1281,12 +1340,16 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_rglru_walk_kernel(const float
 // ------------------------------------------------------------------ gated delta rule
 // After the convolutions: q and k to unit length per head (q also x dim^-1/2), beta =
 // sigmoid, decay g = exp(-exp(a_log) softplus(a + dt_bias)). QKV: [T][ldq] = q | k | v
-// (convolved, silu); Z columns bcol.. = beta logits, acol.. = decay inputs. One workgroup per token.
+// (convolved, silu); Z columns bcol.. = beta logits, acol.. = decay inputs. BG [T][2 H]: beta,
+// per-head decay. GV != nullptr: one decay per head and key channel instead, GV [T][H D] holds
+// the decay inputs on entry (no bias yet; dt_bias is [H D]) and the decays on return, and the
+// per-head decay of BG is 1. One workgroup per token.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_prep_kernel(float *__restrict__ QKV, int ldq, int KH, int D,
                                                                      const float *__restrict__ Z, int ldz, int bcol,
                                                                      int acol, int H, const float *__restrict__ a_log,
                                                                      const float *__restrict__ dt_bias,
-                                                                     float *__restrict__ BG) {
+                                                                     float *__restrict__ BG,
+                                                                     float *__restrict__ GV = nullptr) {
 	const int t = blockIdx.x;
 	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 	float *row = QKV + (size_t)t * ldq;
@@ -1304,8 +1367,29 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_prep_kernel(float *__re
 	for (int h = threadIdx.x; h < H; h += SEQ_THREADS) {
 		BG[(size_t)t * 2 * H + h] = sq_sigmoid(Z[(size_t)t * ldz + bcol + h]);
 		BG[(size_t)t * 2 * H + H + h] =
-		    expf(-expf(a_log[h]) * sq_softplus(Z[(size_t)t * ldz + acol + h] + dt_bias[h]));
+		    GV ? 1.0f : expf(-expf(a_log[h]) * sq_softplus(Z[(size_t)t * ldz + acol + h] + dt_bias[h]));
 	}
+	if (GV)
+		for (int i = threadIdx.x; i < H * D; i += SEQ_THREADS) {
+			float *g = GV + (size_t)t * H * D + i;
+			*g = expf(-expf(a_log[i / D]) * sq_softplus(*g + dt_bias[i]));
+		}
+}
+
+// Selective state-space layer: per token and head dt = softplus(step + dt_bias[h]) and the
+// state's decay exp(-exp(a_log[h]) dt) into BG [T][2 H] (dt, decay), the layout the recurrence
+// kernel reads its per-head factors from. Z columns scol.. = the step inputs.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_ssm_prep_kernel(const float *__restrict__ Z, int ldz, int scol, int H,
+                                                                   const float *__restrict__ a_log,
+                                                                   const float *__restrict__ dt_bias,
+                                                                   float *__restrict__ BG, int T) {
+	const int i = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (i >= T * H)
+		return;
+	const int t = i / H, h = i - t * H;
+	const float dt = sq_softplus(Z[(size_t)t * ldz + scol + h] + dt_bias[h]);
+	BG[(size_t)t * 2 * H + h] = dt;
+	BG[(size_t)t * 2 * H + H + h] = expf(-expf(a_log[h]) * dt);
 }
 
 __device__ __forceinline__ float sum8(float v) { // over aligned groups of 8 lanes
@@ -1322,15 +1406,23 @@ __device__ __forceinline__ float sum8(float v) { // over aligned groups of 8 lan
 // (the read-out after the write). The workgroup's 32 columns share the head's k and q:
 // chunks of TC tokens are staged through two LDS buffers, the next chunk's global loads in
 // flight while the current chunk is applied. grid (ceil(vdim / 32), heads).
-template <int R, int TC>
-__global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__restrict__ QKV, int ldq, int KH, int D,
-                                                                int H, int V, const float *__restrict__ BG,
+// SSM: the state-space form of the same walk, S *= g; S += k (beta v); o = S.q + dskip[h] v
+// (no prediction S.k is taken off the write; k, q, v, beta are the layer's B, C, x and dt).
+// GVEC: g is a vector over the key channels, GV [T][H D], instead of one number per head.
+// QKV [T][ldq]: key/query head kh's q at column qo + kh D, its k at ko + kh D, head h's v at vo + h V.
+template <int R, int TC, bool SSM, bool GVEC>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__restrict__ QKV, int ldq, int qo_, int ko_,
+                                                                int vo_, int KH, int D, int H, int V,
+                                                                const float *__restrict__ BG,
+                                                                const float *__restrict__ GV,
+                                                                const float *__restrict__ dskip,
                                                                 float *__restrict__ state, float *__restrict__ O,
                                                                 int T) {
 	constexpr int DP = 8 * R;                      // padded key dimension
-	constexpr int NKQ = TC * 2 * DP / SEQ_THREADS; // staged k | q values per thread and chunk
+	constexpr int NS = GVEC ? 3 : 2;               // staged rows per token: k | q (| g)
+	constexpr int NKQ = TC * NS * DP / SEQ_THREADS; // staged values per thread and chunk
 	constexpr int COLS = SEQ_THREADS / 8, NV = (TC * COLS + SEQ_THREADS - 1) / SEQ_THREADS;
-	__shared__ __attribute__((aligned(16))) float kq[2][TC][2 * DP];
+	__shared__ __attribute__((aligned(16))) float kq[2][TC][NS * DP];
 	__shared__ float vs[2][TC][COLS], bgs[2][TC][2];
 	const int tid = threadIdx.x;
 	const int h = blockIdx.y, kh = h / (H / KH);
@@ -1342,16 +1434,24 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 #pragma unroll
 	for (int i = 0; i < R; ++i)
 		S[i] = (live && d0 + i < D) ? sp[(size_t)(d0 + i) * V + col] : 0.0f;
-	const int qo = kh * D, ko = KH * D + kh * D, vo = 2 * KH * D + h * V;
+	const int qo = qo_ + kh * D, ko = ko_ + kh * D, vo = vo_ + h * V;
+	const float dsk = (SSM && dskip) ? dskip[h] : 0.0f;
 	// a chunk of TC tokens: global -> registers (in flight while the previous chunk is applied) -> LDS
 	float rkq[NKQ], rv[NV], rbg = 0.0f;
 	auto fetch = [&](int t0) {
 #pragma unroll
 		for (int i = 0; i < NKQ; ++i) {
 			const int idx = tid + i * SEQ_THREADS;
-			const int tt = idx / (2 * DP), e = idx % (2 * DP), d = e % DP;
+			const int tt = idx / (NS * DP), e = idx % (NS * DP), d = e % DP, part = e / DP;
 			const int t = t0 + tt;
-			rkq[i] = (t < T && d < D) ? QKV[(size_t)t * ldq + (e < DP ? ko : qo) + d] : 0.0f;
+			float x = 0.0f;
+			if (t < T && d < D) {
+				if (GVEC && part == 2)
+					x = GV[((size_t)t * H + h) * D + d];
+				else
+					x = QKV[(size_t)t * ldq + (part == 0 ? ko : qo) + d];
+			}
+			rkq[i] = x;
 		}
 #pragma unroll
 		for (int i = 0; i < NV; ++i) {
@@ -1368,7 +1468,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 #pragma unroll
 		for (int i = 0; i < NKQ; ++i) {
 			const int idx = tid + i * SEQ_THREADS;
-			kq[buf][idx / (2 * DP)][idx % (2 * DP)] = rkq[i];
+			kq[buf][idx / (NS * DP)][idx % (NS * DP)] = rkq[i];
 		}
 #pragma unroll
 		for (int i = 0; i < NV; ++i) {
@@ -1388,8 +1488,13 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 		if (more)
 			fetch(t0 + TC);
 		const int nt = min(TC, T - t0);
-		for (int tt = 0; tt < nt; ++tt) {
-			float k[R], q[R];
+		// One token's operands out of LDS, one token ahead of the arithmetic (two register sets in
+		// turn), so that the LDS round trip runs under the previous token's dependent chain.
+		struct Tok {
+			float k[R], q[R], gv[GVEC ? R : 1];
+			float v, beta, g;
+		};
+		auto load = [&](int tt, Tok &x) {
 			if constexpr (R % 4 == 0) {
 #pragma unroll
 				for (int i = 0; i < R / 4; ++i) {
@@ -1397,40 +1502,75 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 					const float4_t q4 = *(const float4_t *)&kq[buf][tt][DP + d0 + 4 * i];
 #pragma unroll
 					for (int e = 0; e < 4; ++e) {
-						k[4 * i + e] = k4[e];
-						q[4 * i + e] = q4[e];
+						x.k[4 * i + e] = k4[e];
+						x.q[4 * i + e] = q4[e];
+					}
+					if constexpr (GVEC) {
+						const float4_t g4 = *(const float4_t *)&kq[buf][tt][2 * DP + d0 + 4 * i];
+#pragma unroll
+						for (int e = 0; e < 4; ++e)
+							x.gv[4 * i + e] = g4[e];
 					}
 				}
 			} else {
 #pragma unroll
 				for (int i = 0; i < R; ++i) {
-					k[i] = kq[buf][tt][d0 + i];
-					q[i] = kq[buf][tt][DP + d0 + i];
+					x.k[i] = kq[buf][tt][d0 + i];
+					x.q[i] = kq[buf][tt][DP + d0 + i];
+					if constexpr (GVEC)
+						x.gv[i] = kq[buf][tt][2 * DP + d0 + i];
 				}
 			}
-			const float v = vs[buf][tt][tid >> 3], beta = bgs[buf][tt][0], g = bgs[buf][tt][1];
+			x.v = vs[buf][tt][tid >> 3];
+			x.beta = bgs[buf][tt][0];
+			x.g = bgs[buf][tt][1];
+		};
+		auto apply = [&](int tt, const Tok &x) {
 			float dd0 = 0.0f, dd1 = 0.0f;
 #pragma unroll
 			for (int i = 0; i < R; ++i) {
-				S[i] *= g;
-				if (i & 1)
-					dd1 = fmaf(S[i], k[i], dd1);
+				if constexpr (GVEC)
+					S[i] *= x.gv[i];
 				else
-					dd0 = fmaf(S[i], k[i], dd0);
+					S[i] *= x.g;
+				if constexpr (!SSM) {
+					if (i & 1)
+						dd1 = fmaf(S[i], x.k[i], dd1);
+					else
+						dd0 = fmaf(S[i], x.k[i], dd0);
+				}
 			}
-			const float u = beta * (v - sum8(dd0 + dd1));
+			float u;
+			if constexpr (SSM)
+				u = x.beta * x.v;
+			else
+				u = x.beta * (x.v - sum8(dd0 + dd1));
 			float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
 			for (int i = 0; i < R; ++i) {
-				S[i] = fmaf(k[i], u, S[i]);
+				S[i] = fmaf(x.k[i], u, S[i]);
 				if (i & 1)
-					o1 = fmaf(S[i], q[i], o1);
+					o1 = fmaf(S[i], x.q[i], o1);
 				else
-					o0 = fmaf(S[i], q[i], o0);
+					o0 = fmaf(S[i], x.q[i], o0);
 			}
-			const float o = sum8(o0 + o1);
+			float o = sum8(o0 + o1);
+			if constexpr (SSM)
+				o = fmaf(dsk, x.v, o);
 			if (sub == 0 && live)
 				O[(size_t)(t0 + tt) * H * V + h * V + col] = o;
+		};
+		Tok xa, xb;
+		load(0, xa);
+		for (int tt = 0; tt < nt; tt += 2) {
+			if (tt + 1 < nt)
+				load(tt + 1, xb);
+			apply(tt, xa);
+			if (tt + 1 < nt) {
+				if (tt + 2 < nt)
+					load(tt + 2, xa);
+				apply(tt + 1, xb);
+			}
 		}
 		if (more)
 			stash(buf ^ 1); // last read while the chunk before this one was applied
@@ -1446,11 +1586,13 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 }
 
 // Each head's read-out divided by its root mean square over vdim, times the shared weight,
-// times silu of the output gate (Z columns gcol..). One workgroup per token, a wave per head.
+// times the output gate: silu (sig == 0) or sigmoid (sig != 0) of the gate logits Gl [t][ldg],
+// head h's at column gcol + h V (out may alias Gl when both rows have the same layout: every
+// entry is read before the same entry is written). One workgroup per token, a wave per head.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_out_kernel(const float *__restrict__ O, int H, int V,
                                                                     const float *__restrict__ w, float eps,
-                                                                    const float *__restrict__ Z, int ldz, int gcol,
-                                                                    float *__restrict__ out) {
+                                                                    const float *Gl, int ldg, int gcol,
+                                                                    float *out, int sig = 0) {
 	const int t = blockIdx.x;
 	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 	for (int h = wave; h < H; h += SEQ_THREADS / 64) {
@@ -1460,10 +1602,31 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_out_kernel(const float 
 			ss = fmaf(o[i], o[i], ss);
 		ss = wave_sum(ss);
 		const float r = 1.0f / sqrtf(ss / (float)V + eps);
-		for (int i = lane; i < V; i += 64)
-			out[(size_t)t * H * V + (size_t)h * V + i] =
-			    o[i] * r * w[i] * sq_silu(Z[(size_t)t * ldz + gcol + h * V + i]);
+		for (int i = lane; i < V; i += 64) {
+			const float gl = Gl[(size_t)t * ldg + gcol + h * V + i];
+			out[(size_t)t * H * V + (size_t)h * V + i] = o[i] * r * w[i] * (sig ? sq_sigmoid(gl) : sq_silu(gl));
+		}
 	}
+}
+
+// Y[t] silu(Z[t][zcol ..]) rms-normed in `parts` equal parts of n / parts entries, each by its own
+// root mean square, times w [n]: out[t]. grid (tokens, parts).
+__global__ __launch_bounds__(SEQ_THREADS) void seq_gated_part_norm_kernel(const float *__restrict__ Y, int n, int parts,
+                                                                          const float *__restrict__ Z, int ldz, int zcol,
+                                                                          const float *__restrict__ w, float eps,
+                                                                          float *__restrict__ out) {
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x, pn = n / parts, c0 = blockIdx.y * pn;
+	const float *y = Y + (size_t)t * n + c0;
+	const float *z = Z + (size_t)t * ldz + zcol + c0;
+	float ss = 0.0f;
+	for (int i = threadIdx.x; i < pn; i += SEQ_THREADS) {
+		const float v = y[i] * sq_silu(z[i]);
+		ss = fmaf(v, v, ss);
+	}
+	const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)pn + eps);
+	for (int i = threadIdx.x; i < pn; i += SEQ_THREADS)
+		out[(size_t)t * n + c0 + i] = y[i] * sq_silu(z[i]) * r * w[c0 + i];
 }
 
 // ------------------------------------------------------------------ latent attention
@@ -1835,8 +1998,10 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_mfma_kernel(const
 // group's score = its best expert's, only experts of the `keep` best groups can be chosen, the
 // `top` largest scores among them win (ties: the lower index); weight = score * rscale, not
 // renormalised. kind 1: the `top` largest logits win (ties: the lower index), weights =
-// softmax over the chosen logits only. Also the shared expert's gate sigmoid(w_sg . h).
-// Dynamic LDS: E + G floats.
+// softmax over the chosen logits only. kind 2: scores sigmoid(logit); the choice ranks score +
+// bias: a group by the sum of its two largest, the `top` largest within the `keep` best groups
+// win (ties: the lower index); weight = score * rscale, without the bias, not renormalised.
+// Also the shared expert's gate sigmoid(w_sg . h). Dynamic LDS: 2 E + G floats.
 #define SEQ_MAX_GROUPS 64
 __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__restrict__ Hn, int width,
                                                                  const float *__restrict__ Wr, int E, int top, int G,
@@ -1869,7 +2034,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__
 		a = wave_sum(a);
 		if (lane == 0) {
 			if (e < E)
-				sc[e] = a + (bias ? bias[e] : 0.0f);
+				sc[e] = a + ((bias && kind != 2) ? bias[e] : 0.0f);
 			else
 				sgate[t] = sq_sigmoid(a);
 		}
@@ -1901,6 +2066,53 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__
 	}
 	float *gsc = sc + E; // [G]
 	__shared__ float red[SEQ_THREADS / 64];
+	if (kind == 2) { // sc holds the logits (no bias added above)
+		if (threadIdx.x != 0)
+			return;
+		const int gs = E / G;
+		float *sv = gsc + G; // [E] the scores themselves (the weights); sc becomes the choice scores
+		for (int e = 0; e < E; ++e) {
+			sv[e] = sq_sigmoid(sc[e]);
+			sc[e] = sv[e] + (bias ? bias[e] : 0.0f);
+		}
+		for (int g = 0; g < G; ++g) { // sum of the group's two largest choice scores
+			float m1 = -INFINITY, m2 = -INFINITY;
+			for (int e = g * gs; e < (g + 1) * gs; ++e) {
+				const float v = sc[e];
+				if (v > m1) {
+					m2 = m1;
+					m1 = v;
+				} else if (v > m2) {
+					m2 = v;
+				}
+			}
+			gsc[g] = gs > 1 ? m1 + m2 : m1;
+		}
+		unsigned long long allowed = 0ull;
+		for (int k = 0; k < keep; ++k) {
+			int best = -1;
+			float bv = -INFINITY;
+			for (int g = 0; g < G; ++g)
+				if (!((allowed >> g) & 1ull) && (best < 0 || gsc[g] > bv)) {
+					bv = gsc[g];
+					best = g;
+				}
+			allowed |= 1ull << best;
+		}
+		for (int k = 0; k < top; ++k) {
+			int best = -1;
+			float bv = -INFINITY;
+			for (int e = 0; e < E; ++e)
+				if (((allowed >> (e / gs)) & 1ull) && sc[e] != -INFINITY && (best < 0 || sc[e] > bv)) {
+					bv = sc[e];
+					best = e;
+				}
+			idx[(size_t)t * top + k] = best;
+			wt[(size_t)t * top + k] = sv[best] * rscale;
+			sc[best] = -INFINITY; // taken
+		}
+		return;
+	}
 	float mx = -FLT_MAX;
 	for (int e = threadIdx.x; e < E; e += SEQ_THREADS)
 		mx = fmaxf(mx, sc[e]);

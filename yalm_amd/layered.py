@@ -6,9 +6,11 @@ description; a design registers a reader that turns its ``config.json`` into one
 a packer that turns its checkpoint tensors into the engine's per-layer tensors
 (concatenated input projections, per-head transposed key up-projections, stacked
 experts). ``Sinulorn`` (latent attention, recurrences, routed experts), ``Lenuzen``
-(windowed / chunked softmax attention, plain feed-forwards) and ``Mirorax`` (parallel
+(windowed / chunked softmax attention, plain feed-forwards), ``Mirorax`` (parallel
 blocks with layer scales, a looped run of layers, gated attention, latent attention with a
-rotated key part, a window and a learned sink) are such designs.
+rotated key part, a window and a learned sink) and ``Lifenex`` (parallel blocks with a norm
+per sublayer, a selective state-space mixer, attention with a distance bias beside a delta
+rule with per-channel decays, grouped sigmoid routing) are such designs.
 
 Checkpoints are folders with ``config.json`` and ``model.safetensors`` (bf16
 matrices; read with yalmfile.read_yalm, the same container the .yalm files use).
@@ -24,14 +26,15 @@ import numpy as np
 
 from . import models as M
 
-MIX_LATENT, MIX_RGLRU, MIX_DELTA, MIX_ATTN = 0, 1, 2, 3
+MIX_LATENT, MIX_RGLRU, MIX_DELTA, MIX_ATTN, MIX_SSM = 0, 1, 2, 3, 4
 FF_NONE, FF_DENSE, FF_MOE, FF_PLAIN = 0, 1, 2, 3
 NORM_RMS, NORM_LAYER = 0, 1
 MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
-QK_NONE, QK_HEAD_UNIT, QK_WHOLE = 0, 1, 2
+QK_NONE, QK_HEAD_UNIT, QK_WHOLE, QK_HEAD_W = 0, 1, 2, 3
 BLOCK_SERIAL, BLOCK_PARALLEL = 0, 1
-ACT_DEFAULT, ACT_GELU, ACT_CLAMP, ACT_SILU = 0, 1, 2, 3
-ROUTER_SOFTMAX_TOP, ROUTER_TOP_SOFTMAX = 0, 1
+ACT_DEFAULT, ACT_GELU, ACT_CLAMP, ACT_SILU, ACT_RELU2 = 0, 1, 2, 3, 4
+ROUTER_SOFTMAX_TOP, ROUTER_TOP_SOFTMAX, ROUTER_SIGMOID_GROUPS = 0, 1, 2
+DELTA_GATE_SILU, DELTA_GATE_SIGMOID = 0, 1
 GATE_NONE, GATE_HEAD, GATE_ELEMENT = 0, 1, 2
 
 
@@ -88,6 +91,26 @@ class LayerSpec:
     # layer runs
     pre_added: bool = False     # a vector joins the stream before this run's opening norm
     shares: int = -1            # >= 0: this run uses the tensors of that (earlier) run, all but pre_add
+    # selective state-space mixer: heads x vdim channels, a state of ssm_state x vdim per head
+    ssm_state: int = 0
+    ssm_groups: int = 1
+    norm_groups: int = 1
+    # delta rule: low-rank decay per head and key channel / low-rank output gate (0: the plain forms)
+    decay_rank: int = 0
+    gate_rank: int = 0
+    gate_act: int = DELTA_GATE_SILU
+    # softmax attention: query temperature by position, learned bias per head and bucketed distance
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 0
+    rel_rows: int = 0
+    rel_max: float = 0.0
+    # a second mixer beside this one (a LayerSpec whose mixer fields alone are used); the two
+    # results are rms-normed with join_w / side_join_w, summed and scaled by join_scale
+    side: "LayerSpec" = None
+    join_scale: float = 1.0
+    # parallel blocks: the feed-forward reads its own norm (norm2) of the stream; no layer scales
+    ff_normed: bool = False
+    layer_scaled: bool = True
 
     @property
     def in_rows(self) -> int:
@@ -101,7 +124,10 @@ class LayerSpec:
         if self.mixer == MIX_ATTN:
             gate = {GATE_NONE: 0, GATE_HEAD: self.heads, GATE_ELEMENT: self.heads * self.vdim}[self.out_gate]
             return self.heads * self.dim + self.kv_heads * (self.dim + self.vdim) + gate
-        return 2 * self.kv_heads * self.dim + 2 * self.heads * self.vdim + 2 * self.heads
+        if self.mixer == MIX_SSM:
+            return 2 * self.heads * self.vdim + 2 * self.ssm_groups * self.ssm_state + self.heads
+        return (2 * self.kv_heads * self.dim + self.heads * self.vdim + (self.gate_rank or self.heads * self.vdim)
+                + self.heads + (self.decay_rank or self.heads))
 
     @property
     def mix_out(self) -> int:
@@ -125,24 +151,32 @@ class LayeredConfig:
     logit_scale: float = 1.0
     tied_head: bool = False   # the logits read the embedding table
     block_kind: int = BLOCK_SERIAL  # BLOCK_PARALLEL: x += ls1 * mixer(norm1(x)) + ls2 * ff(norm1(x))
+    embed_normed: bool = False  # the embedding row is rms-normed (weight embed_norm) before it becomes the stream
 
     def with_(self, **kw) -> "LayeredConfig":
         return dataclasses.replace(self, **kw)
 
 
-def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
+def packed_shapes(c: LayeredConfig, l: LayerSpec, side: bool = False) -> dict:
     """field -> (shape, kind) of one layer's engine tensors; kind "w": a matrix of the
-    model's weight dtype, "f": f32."""
+    model's weight dtype, "f": f32. side: l is a layer's second mixer (its mixer tensors only)."""
     W = c.width
     out = {}
     if l.pre_added:
         out["pre_add"] = ((W,), "f")
     if l.shares >= 0:
         return out
-    if c.block_kind == BLOCK_PARALLEL:
-        out["norm1"] = out["ls1"] = ((W,), "f")
+    if side:
+        pass
+    elif c.block_kind == BLOCK_PARALLEL:
+        out["norm1"] = ((W,), "f")
+        if l.layer_scaled:
+            out["ls1"] = ((W,), "f")
         if l.ff_kind != FF_NONE:
-            out["ls2"] = ((W,), "f")
+            if l.layer_scaled:
+                out["ls2"] = ((W,), "f")
+            if l.ff_normed:
+                out["norm2"] = ((W,), "f")
     else:
         out["norm1b"] = ((W,), "f")
         if c.pre_norm:
@@ -151,6 +185,8 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
             out["norm2b"] = ((W,), "f")
             if c.pre_norm:
                 out["norm2"] = ((W,), "f")
+    if l.side is not None:
+        out["join_w"] = out["side_join_w"] = ((W,), "f")
     out["w_in"] = ((l.in_rows, W), "w")
     out["w_o"] = ((W, l.mix_out), "w")
     if l.o_biased:
@@ -184,10 +220,22 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
             out["head_temp"] = ((l.heads,), "f")
         if l.talking:
             out["talk"] = ((l.heads, l.heads), "f")
+        if l.qk_norm == QK_HEAD_W:
+            out.update(q_norm=((l.dim,), "f"), kv_norm=((l.dim,), "f"))
+        if l.rel_rows:
+            out["rel"] = ((l.rel_rows, l.heads), "f")
+    elif l.mixer == MIX_SSM:
+        inner, cc = l.heads * l.vdim, l.heads * l.vdim + 2 * l.ssm_groups * l.ssm_state
+        out.update(conv_w=((cc, l.conv), "f"), conv_b=((cc,), "f"), a_log=((l.heads,), "f"), dt_bias=((l.heads,), "f"),
+                   d_skip=((l.heads,), "f"), out_norm=((inner,), "f"))
     else:
         cc = 2 * l.kv_heads * l.dim + l.heads * l.vdim
-        out.update(conv_w=((cc, l.conv), "f"), a_log=((l.heads,), "f"), dt_bias=((l.heads,), "f"),
-                   out_norm=((l.vdim,), "f"))
+        out.update(conv_w=((cc, l.conv), "f"), a_log=((l.heads,), "f"),
+                   dt_bias=((l.heads * l.dim if l.decay_rank else l.heads,), "f"), out_norm=((l.vdim,), "f"))
+        if l.decay_rank:
+            out["w_a2"] = ((l.heads * l.dim, l.decay_rank), "w")
+        if l.gate_rank:
+            out["w_g2"] = ((l.heads * l.vdim, l.gate_rank), "w")
     if l.ff_kind == FF_PLAIN:
         out.update(w_up=((l.ff, W), "w"), w_down=((W, l.ff), "w"))
     if l.ff_kind == FF_DENSE:
@@ -751,10 +799,230 @@ def mirorax_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0) -> dict:
     return out
 
 
+# ------------------------------------------------------------------ Lifenex
+# x = rms(E[token]) w_e. Every layer is a parallel block with a norm per sublayer: x += mixer(rms(x)
+# w1) + ff(rms(x) w2). Two mixers:
+#   "mamba2":   a selective state-space layer: W_in h = [gate | x | B | C | step]; x | B | C pass a
+#               biased causal convolution and silu; per head dt = softplus(step + dt_bias), S <-
+#               exp(-exp(A) dt) S + dt B x^T, y = S^T C + D x; y silu(gate) rms-normed in norm_groups
+#               equal parts; W_o;
+#   "parallel": two mixers on the same input, result = (rms(left) w_l + rms(right) w_r) / 2:
+#               left, softmax attention without rotation (per-head weighted rms norm of queries and
+#               keys, query temperature 1 + coef ln(floor((p + 1) / every) + 1), a learned bias per
+#               head and bucketed distance added to the scaled score, a learned sink in the
+#               denominator); right, a gated delta rule with one decay per head and key channel
+#               (low-rank decay and gate projections, sigmoid output gate).
+# Feed-forwards: "dense" W_d relu(W_u h)^2; "moe": silu-gated experts, scores sigmoid(W_r h), the
+# choice by score + correction within the best groups (a group's rank: the sum of its two best),
+# weights the plain scores, plus a shared expert times sigmoid(w_sg . h). Logits: the embedding
+# table on the final norm, times logit_scale.
+LIFENEX_MIXERS = ("mamba2", "parallel")
+
+
+def _lifenex_layer(e: dict) -> LayerSpec:
+    m = e["mixer"]
+    if e["type"] == "mamba2":
+        s = LayerSpec(MIX_SSM, heads=m["heads"], vdim=m["vdim"], ssm_state=m["state"], ssm_groups=m.get("groups", 1),
+                      norm_groups=m.get("norm_groups", 1), conv=m["conv"])
+    elif e["type"] == "parallel":
+        a, d = m["left"], m["right"]
+        qt = a.get("q_temp") or {}
+        s = LayerSpec(MIX_ATTN, heads=a["heads"], kv_heads=a.get("kv_heads", a["heads"]), dim=a["dim"], vdim=a["vdim"],
+                      attn_scale=float(a["scale"]), mask_kind=MASK_CAUSAL, qk_norm=QK_HEAD_W, sink=1, sink_learned=True,
+                      q_temp_coef=float(qt.get("coef", 0.0)), q_temp_every=int(qt.get("every", 0)),
+                      rel_max=float(a["bias_max"]), rel_rows=-1, join_scale=0.5)
+        s.side = LayerSpec(MIX_DELTA, heads=d["heads"], kv_heads=d.get("kv_heads", d["heads"]), dim=d["dim"],
+                           vdim=d["vdim"], conv=d["conv"], decay_rank=-1, gate_rank=-1, gate_act=DELTA_GATE_SIGMOID)
+    else:
+        raise ValueError(f"unknown mixer type {e['type']!r}")
+    s.ff_normed, s.layer_scaled = True, False
+    mlp = e.get("mlp")
+    if mlp:
+        if mlp["kind"] == "dense":
+            s.ff_kind, s.ff, s.ff_act = FF_PLAIN, mlp["ff"], ACT_RELU2
+        elif mlp["kind"] == "moe":
+            r = mlp["router"]
+            g = r.get("groups") or {"count": 1, "keep": 1}
+            s.ff_kind, s.ff, s.ff_act = FF_MOE, mlp["expert"]["ff"], ACT_SILU
+            s.experts, s.top, s.groups, s.groups_keep = r["experts"], r["top"], g["count"], g["keep"]
+            s.router_kind, s.router_biased, s.router_scale = ROUTER_SIGMOID_GROUPS, True, 1.0
+            if mlp.get("shared"):
+                s.shared_ff, s.shared_gated = mlp["shared"]["ff"], True
+        else:
+            raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+    return s
+
+
+def lifenex_config(cfg: dict, max_tokens: int = 4096, weight_dtype: int = M.BF16, shapes: dict = None) -> LayeredConfig:
+    """config.json of a Lifenex checkpoint -> LayeredConfig. Every size and every constant that
+    can differ between models of the design is read from cfg; the sizes config.json does not
+    name (rows of the distance-bias table, ranks of the low-rank decay and gate) are the
+    checkpoint tensors' own: shapes maps tensor names to shapes."""
+    layers = []
+    for i, e in enumerate(cfg["layers"]):
+        s = _lifenex_layer(e)
+        if s.side is not None:
+            if shapes is None:
+                raise ValueError("a Lifenex 'parallel' layer takes sizes from the checkpoint's tensor shapes")
+            s.rel_rows = int(shapes[f"l{i}.mix.left.rel"][0])
+            s.side.decay_rank = int(shapes[f"l{i}.mix.right.a1"][0])
+            s.side.gate_rank = int(shapes[f"l{i}.mix.right.g1"][0])
+        layers.append(s)
+    return LayeredConfig(
+        arch="Lifenex", width=cfg["width"], vocab=cfg["vocab"], layers=layers, embed_scale=1.0,
+        norm_eps=float(cfg["norm"]["eps"]), max_tokens=max_tokens, weight_dtype=weight_dtype, norm_kind=NORM_RMS,
+        pre_norm=True, pos_embed=False, logit_scale=float(cfg.get("logit_scale", 1.0)), tied_head=True,
+        block_kind=BLOCK_PARALLEL, embed_normed=True,
+    )
+
+
+def lifenex_tensor_shapes(cfg: dict, rel_rows: int = 16, decay_rank: int = 8, gate_rank: int = 8) -> dict:
+    """Checkpoint tensor name -> shape for a Lifenex config.json; the three sizes config.json
+    does not name are arguments."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W), "embed.norm": (W,), "final.norm": (W,)}
+    for i, e in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", e["mixer"]
+        x = p + "mix."
+        out[p + "norm1"] = (W,)
+        if e["type"] == "mamba2":
+            H, P, N, G = m["heads"], m["vdim"], m["state"], m.get("groups", 1)
+            inner, cc = H * P, H * P + 2 * G * N
+            out[x + "in"], out[x + "conv"], out[x + "conv.b"] = (2 * inner + 2 * G * N + H, W), (cc, m["conv"]), (cc,)
+            out[x + "dt_bias"] = out[x + "A_log"] = out[x + "D"] = (H,)
+            out[x + "norm"], out[x + "o"] = (inner,), (W, inner)
+        else:
+            a, d = m["left"], m["right"]
+            H, G, D, V = a["heads"], a.get("kv_heads", a["heads"]), a["dim"], a["vdim"]
+            y = x + "left."
+            out[y + "q"], out[y + "k"], out[y + "v"], out[y + "o"] = (H * D, W), (G * D, W), (G * V, W), (W, H * V)
+            out[y + "q.norm"] = out[y + "k.norm"] = (D,)
+            out[y + "rel"], out[y + "sink"] = (rel_rows, H), (H,)
+            H, KH, D, V = d["heads"], d.get("kv_heads", d["heads"]), d["dim"], d["vdim"]
+            y = x + "right."
+            for n, rows in (("q", KH * D), ("k", KH * D), ("v", H * V)):
+                out[y + n], out[y + n + ".conv"] = (rows, W), (rows, d["conv"])
+            out[y + "b"], out[y + "A_log"], out[y + "norm"] = (H, W), (H,), (V,)
+            out[y + "a1"], out[y + "a2"], out[y + "dt_bias"] = (decay_rank, W), (H * D, decay_rank), (H * D,)
+            out[y + "g1"], out[y + "g2"], out[y + "o"] = (gate_rank, W), (H * V, gate_rank), (W, H * V)
+            out[x + "left.out"] = out[x + "right.out"] = (W,)
+        mlp = e.get("mlp")
+        if not mlp:
+            continue
+        out[p + "norm2"] = (W,)
+        f = p + "mlp."
+        if mlp["kind"] == "dense":
+            out[f + "up"], out[f + "down"] = (mlp["ff"], W), (W, mlp["ff"])
+        else:
+            ff, E = mlp["expert"]["ff"], mlp["router"]["experts"]
+            for k in range(E):
+                out[f"{f}e{k}.gate"] = out[f"{f}e{k}.up"] = (ff, W)
+                out[f"{f}e{k}.down"] = (W, ff)
+            out[f + "router"], out[f + "correction"] = (E, W), (E,)
+            if mlp.get("shared"):
+                sf = mlp["shared"]["ff"]
+                out[f + "shared.gate"] = out[f + "shared.up"] = (sf, W)
+                out[f + "shared.down"], out[f + "shared.sg"] = (W, sf), (1, W)
+    return out
+
+
+def _check_packed(where: str, want: dict, d: dict) -> None:
+    if set(want) != set(d):
+        raise ValueError(f"{where}: packed tensors {sorted(d)} do not match the configuration's {sorted(want)}")
+    for k, (shape, _) in want.items():
+        if tuple(d[k].shape) != tuple(shape):
+            raise ValueError(f"{where}: tensor {k} has shape {d[k].shape}, the configuration gives {shape}")
+
+
+def lifenex_pack(c: LayeredConfig, t: dict) -> dict:
+    """Checkpoint tensors -> the engine's tensors (see sinulorn_pack). The input projections of a
+    mixer become one w_in (attention: q | k | v; delta rule: q | k | v | gate down | beta | decay
+    down); a layer's second mixer is the nested dict "side"."""
+    dt = c.weight_dtype
+
+    def w(*names):
+        parts = [_as_weight(t[n], dt) for n in names]
+        return parts[0] if len(parts) == 1 else np.ascontiguousarray(np.concatenate(parts, axis=0))
+
+    def f(name):
+        return np.ascontiguousarray(_as_f32(t[name]))
+
+    layers = []
+    for i, l in enumerate(c.layers):
+        p, x, m = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        d = {"norm1": f(p + "norm1")}
+        if l.mixer == MIX_SSM:
+            d.update(w_in=w(x + "in"), conv_w=f(x + "conv"), conv_b=f(x + "conv.b"), a_log=f(x + "A_log"),
+                     dt_bias=f(x + "dt_bias"), d_skip=f(x + "D"), out_norm=f(x + "norm"), w_o=w(x + "o"))
+        else:
+            y = x + "left."
+            d.update(w_in=w(y + "q", y + "k", y + "v"), q_norm=f(y + "q.norm"), kv_norm=f(y + "k.norm"),
+                     rel=f(y + "rel"), sink_w=f(y + "sink"), w_o=w(y + "o"), join_w=f(x + "left.out"),
+                     side_join_w=f(x + "right.out"))
+            y = x + "right."
+            sd = {"w_in": w(y + "q", y + "k", y + "v", y + "g1", y + "b", y + "a1"),
+                  "conv_w": np.ascontiguousarray(np.concatenate([f(y + n + ".conv") for n in ("q", "k", "v")], axis=0)),
+                  "a_log": f(y + "A_log"), "dt_bias": f(y + "dt_bias"), "out_norm": f(y + "norm"),
+                  "w_a2": w(y + "a2"), "w_g2": w(y + "g2"), "w_o": w(y + "o")}
+            _check_packed(f"layer {i}, second mixer", packed_shapes(c, l.side, side=True), sd)
+        if l.ff_kind != FF_NONE:
+            d["norm2"] = f(p + "norm2")
+        if l.ff_kind == FF_PLAIN:
+            d.update(w_up=w(m + "up"), w_down=w(m + "down"))
+        elif l.ff_kind == FF_MOE:
+            d.update(router=f(m + "router"), router_bias=f(m + "correction"))
+            for k in ("gate", "up", "down"):
+                d["w_" + k] = np.ascontiguousarray(
+                    np.stack([_as_weight(t[f"{m}e{e}.{k}"], dt) for e in range(l.experts)]))
+            if l.shared_ff:
+                d.update(ws_gate=w(m + "shared.gate"), ws_up=w(m + "shared.up"), ws_down=w(m + "shared.down"),
+                         shared_sg=f(m + "shared.sg").reshape(-1))
+        _check_packed(f"layer {i}", packed_shapes(c, l), d)
+        if l.side is not None:
+            d["side"] = sd
+        layers.append(d)
+    emb = w("embed")
+    return {"embed": emb, "embed_norm": f("embed.norm"), "final_norm": f("final.norm"), "head": emb, "layers": layers}
+
+
+def lifenex_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0, **sizes) -> dict:
+    """Random checkpoint tensors for a Lifenex config.json, as float32 arrays already rounded to
+    bf16 values (the f32 and bf16 engines and a float64 restatement see the same weights)."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in lifenex_tensor_shapes(cfg, **sizes).items():
+        leaf = name.split(".")[-1]
+        if leaf in ("norm1", "norm2", "out") or name.endswith(".norm"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif leaf == "b" and len(shape) == 1:
+            a = 0.3 * rng.standard_normal(shape)
+        elif leaf == "conv":
+            a = 0.5 * rng.standard_normal(shape)
+        elif leaf == "A_log":
+            a = rng.uniform(-3.0, 0.5, shape)
+        elif leaf == "dt_bias":
+            a = rng.uniform(-2.0, 1.0, shape)
+        elif leaf == "D":
+            a = rng.uniform(0.5, 1.5, shape)
+        elif leaf == "rel":
+            a = 0.7 * rng.standard_normal(shape)
+        elif leaf == "sink":
+            a = rng.uniform(-1.0, 2.0, shape)
+        elif leaf == "correction":
+            a = 0.2 * rng.standard_normal(shape)
+        elif leaf == "embed":
+            a = 0.5 * rng.standard_normal(shape)
+        else:
+            a = gain * rng.standard_normal(shape) / np.sqrt(shape[-1])
+        out[name] = bf16_to_f32(f32_to_bf16(a.astype(np.float32))).reshape(shape)
+    return out
+
+
 # ------------------------------------------------------------------ registry
 # design name (config.json "architecture") -> (config reader, weight packer)
 DESIGNS = {"Sinulorn": (sinulorn_config, sinulorn_pack), "Lenuzen": (lenuzen_config, lenuzen_pack),
-           "Mirorax": (mirorax_config, lambda c, t, cfg=None: mirorax_pack(c, t, cfg))}
+           "Mirorax": (mirorax_config, lambda c, t, cfg=None: mirorax_pack(c, t, cfg)),
+           "Lifenex": (lifenex_config, lifenex_pack)}
 
 
 def read_checkpoint(path: str, max_tokens: int = 4096, weight_dtype: int = M.BF16):
@@ -768,9 +1036,12 @@ def read_checkpoint(path: str, max_tokens: int = 4096, weight_dtype: int = M.BF1
     if arch not in DESIGNS:
         raise ValueError(f"architecture {arch!r} is not a layer-list design this engine knows ({sorted(DESIGNS)})")
     reader, packer = DESIGNS[arch]
-    c = reader(cfg, max_tokens, weight_dtype)
     yd = read_yalm(os.path.join(path, "model.safetensors"))
     try:
+        if arch == "Lifenex":  # some sizes are the tensors' own
+            c = reader(cfg, max_tokens, weight_dtype, {k: tuple(v.shape) for k, v in yd.tensors.items()})
+        else:
+            c = reader(cfg, max_tokens, weight_dtype)
         t = {k: np.asarray(v.data).reshape(v.shape) for k, v in yd.tensors.items()}
         return c, (packer(c, t, cfg) if arch == "Mirorax" else packer(c, t))
     finally:

@@ -145,7 +145,8 @@ class SeqLayer(ctypes.Structure):
     PTRS = ("norm1", "norm1b", "norm2", "norm2b", "ls1", "ls2", "pre_add", "sink_w", "o_bias", "router_bias",
             "q_norm", "kv_norm", "in_bias", "head_temp", "talk", "conv_w", "conv_b", "gate_a",
             "gate_a_b", "gate_i", "gate_i_b", "lam", "a_log", "dt_bias", "out_norm", "router", "shared_sg",
-            "w_in", "w_uq", "w_ukt", "w_uv", "w_ukv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
+            "w_in", "w_uq", "w_ukt", "w_uv", "w_ukv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down",
+            "rel", "d_skip", "join_w", "side_join_w", "w_a2", "w_g2", "side")
     _fields_ = (
         [(n, c_int) for n in INTS] + [("attn_scale", c_float), ("rec_width", c_int), ("blocks", c_int), ("conv", c_int),
                                       ("ff_kind", c_int), ("ff", c_int), ("experts", c_int), ("top", c_int),
@@ -155,6 +156,9 @@ class SeqLayer(ctypes.Structure):
         + [(n, c_int) for n in ("mask_kind", "mask_size", "qk_norm", "v_norm", "sink", "out_gate", "rot_dims",
                                 "rot_orig")]
         + [(n, c_float) for n in ("rot_base", "rot_factor", "rot_fast", "rot_slow")]
+        + [(n, c_int) for n in ("ssm_state", "ssm_groups", "norm_groups", "decay_rank", "gate_rank", "gate_act")]
+        + [("q_temp_coef", c_float), ("q_temp_every", c_int), ("rel_rows", c_int), ("rel_max", c_float),
+           ("join_scale", c_float)]
         + [(n, c_void_p) for n in PTRS]
     )
 
@@ -166,7 +170,8 @@ class SeqConfig(ctypes.Structure):
 
 
 class SeqWeights(ctypes.Structure):
-    _fields_ = [("embed", c_void_p), ("final_norm", c_void_p), ("head", c_void_p), ("layers", ctypes.POINTER(SeqLayer))]
+    _fields_ = [("embed", c_void_p), ("final_norm", c_void_p), ("head", c_void_p), ("layers", ctypes.POINTER(SeqLayer)),
+                ("embed_norm", c_void_p)]
 
 
 _sig("yalm_seq_create", c_int, [ctypes.POINTER(SeqConfig), ctypes.POINTER(SeqWeights), c_void_p,
@@ -661,14 +666,23 @@ class SeqModel:
         for k in ("embed", "final_norm", "head"):
             # a tied head aliases the embedding table instead of a second upload
             self.ptrs[k] = self.ptrs["embed"] if k == "head" and packed[k] is packed["embed"] else self._up(packed[k])
+        if packed.get("embed_norm") is not None:
+            self.ptrs["embed_norm"] = self._up(packed["embed_norm"])
         seen = {}  # layer runs that share tensors hold the same arrays: one upload each
-        for d in packed["layers"]:
+
+        def up(d):
             ptrs = {}
             for k, a in d.items():
+                if k == "side":  # the layer's second mixer: a dict of its own tensors
+                    ptrs[k] = up(a)
+                    continue
                 if id(a) not in seen:
                     seen[id(a)] = self._up(a)
                 ptrs[k] = seen[id(a)]
-            self.layer_ptrs.append(ptrs)
+            return ptrs
+
+        for d in packed["layers"]:
+            self.layer_ptrs.append(up(d))
         return self
 
     @classmethod
@@ -698,7 +712,8 @@ class SeqModel:
             leaf = name.rsplit(".", 1)[-1]
             if kind == "w" or leaf in ("router", "gate_a", "gate_i", "shared_sg"):
                 scale, off = 1.7 / np.sqrt(fan_in or shape[-1]), 0.0
-            elif leaf.startswith("norm") or leaf in ("q_norm", "kv_norm", "out_norm", "final_norm", "head_temp"):
+            elif leaf.startswith("norm") or leaf in ("q_norm", "kv_norm", "out_norm", "final_norm", "head_temp",
+                                                     "embed_norm", "join_w", "side_join_w", "d_skip"):
                 scale, off = 0.2, 1.0
             elif leaf in ("ls1", "ls2"):
                 scale, off = 0.2, 0.6
@@ -714,8 +729,13 @@ class SeqModel:
         self.ptrs["embed"] = make("embed", (cfg.vocab, cfg.width), "w", fan_in=100.0)
         self.ptrs["final_norm"] = make("final_norm", (cfg.width,), "f")
         self.ptrs["head"] = self.ptrs["embed"] if cfg.tied_head else make("head", (cfg.vocab, cfg.width), "w")
+        if cfg.embed_normed:
+            self.ptrs["embed_norm"] = make("embed_norm", (cfg.width,), "f")
         for i, l in enumerate(cfg.layers):
             ptrs = {k: make(f"l{i}.{k}", shape, kind) for k, (shape, kind) in layered.packed_shapes(cfg, l).items()}
+            if l.side is not None:
+                ptrs["side"] = {k: make(f"l{i}.side.{k}", shape, kind)
+                                for k, (shape, kind) in layered.packed_shapes(cfg, l.side, side=True).items()}
             if l.shares >= 0:  # a repeated run: the first pass's tensors, its own pre_add
                 ptrs = {**{k: v for k, v in self.layer_ptrs[l.shares].items() if k != "pre_add"}, **ptrs}
             self.layer_ptrs.append(ptrs)
@@ -725,16 +745,30 @@ class SeqModel:
     def structs(self):
         cfg = self.cfg
         arr = (SeqLayer * len(cfg.layers))()
-        for i, (l, ptrs) in enumerate(zip(cfg.layers, self.layer_ptrs)):
+        n_sides = sum(l.side is not None for l in cfg.layers)
+        sides = (SeqLayer * max(n_sides, 1))()  # the layers' second mixers; `arr` points into it
+
+        def fill(dst, l, ptrs):
             for name, _ in SeqLayer._fields_:
+                if name == "side":
+                    continue
                 if name in SeqLayer.PTRS:
-                    setattr(arr[i], name, ptrs.get(name))
+                    setattr(dst, name, ptrs.get(name))
                 else:
-                    setattr(arr[i], name, getattr(l, name))
+                    setattr(dst, name, getattr(l, name))
+
+        k = 0
+        for i, (l, ptrs) in enumerate(zip(cfg.layers, self.layer_ptrs)):
+            fill(arr[i], l, ptrs)
+            if l.side is not None:
+                fill(sides[k], l.side, ptrs["side"])
+                arr[i].side = ctypes.addressof(sides[k])
+                k += 1
+        arr._sides = sides  # kept alive with the layer array
         sc = SeqConfig(cfg.width, cfg.vocab, len(cfg.layers), cfg.max_tokens, cfg.embed_scale, cfg.norm_eps,
                        cfg.weight_dtype, cfg.norm_kind, int(cfg.pre_norm), int(cfg.pos_embed), cfg.logit_scale,
                        cfg.block_kind)
-        sw = SeqWeights(self.ptrs["embed"], self.ptrs["final_norm"], self.ptrs["head"], arr)
+        sw = SeqWeights(self.ptrs["embed"], self.ptrs["final_norm"], self.ptrs["head"], arr, self.ptrs.get("embed_norm"))
         return sc, sw, arr
 
     def close(self):
