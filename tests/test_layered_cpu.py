@@ -296,7 +296,7 @@ def test_bench_stacks_are_valid_layer_list_configurations():
     import bench
 
     for width in (1024, 2048, 4096):
-        for make in (bench.layered_stack, bench.lenuzen_stack, bench.mirorax_stack):
+        for make in (bench.layered_stack, bench.lenuzen_stack, bench.mirorax_stack, bench.lifenex_stack):
             c = make(Ly, M, width, 2112)
             assert c.width == width and len(c.layers) == 6
             for l in c.layers:
@@ -305,9 +305,126 @@ def test_bench_stacks_are_valid_layer_list_configurations():
                     assert set(shapes) <= {"pre_add"} and c.layers[l.shares].mixer == l.mixer
                     continue
                 assert shapes["w_in"][0] == (l.in_rows, width) and shapes["w_o"][0] == (width, l.mix_out)
+                if l.side is not None:
+                    side = Ly.packed_shapes(c, l.side, side=True)
+                    assert side["w_in"][0] == (l.side.in_rows, width) and "norm1" not in side and "join_w" in shapes
                 if l.mixer == Ly.MIX_ATTN:
                     assert l.heads % l.kv_heads == 0 and l.rot_dims <= l.dim
                     if l.talking:
                         assert l.kv_heads * l.dim <= 512 and "talk" in shapes
     c = bench.lenuzen_stack(Ly, M, 2048, 2112)
     assert (c.norm_kind, c.pre_norm, c.pos_embed, c.tied_head) == (Ly.NORM_LAYER, False, False, True)
+
+
+# ------------------------------------------------------------------ Lifenex
+def test_lifenex_config_reads_every_size_and_constant():
+    import lifenex_cases as LC
+
+    cfg = LC.MIXED
+    t = Ly.lifenex_random_tensors(cfg, seed=1, **LC.sizes(cfg))
+    c = Ly.lifenex_config(cfg, max_tokens=99, weight_dtype=M.F32, shapes={k: v.shape for k, v in t.items()})
+    assert (c.arch, c.width, c.vocab, c.max_tokens, c.weight_dtype) == ("Lifenex", 96, 211, 99, M.F32)
+    assert (c.block_kind, c.pre_norm, c.pos_embed, c.tied_head, c.embed_normed) == (Ly.BLOCK_PARALLEL, True, False, True, True)
+    assert c.logit_scale == 0.5 and c.norm_eps == 1e-5 and c.norm_kind == Ly.NORM_RMS
+    s0, m0 = c.layers[0], cfg["layers"][0]["mixer"]
+    assert (s0.mixer, s0.heads, s0.vdim, s0.ssm_state, s0.ssm_groups, s0.norm_groups, s0.conv) == (
+        Ly.MIX_SSM, m0["heads"], m0["vdim"], m0["state"], m0["groups"], m0["norm_groups"], m0["conv"])
+    assert (s0.ff_kind, s0.ff, s0.ff_act, s0.ff_normed, s0.layer_scaled) == (Ly.FF_PLAIN, 72, Ly.ACT_RELU2, True, False)
+    s2, m2 = c.layers[2], cfg["layers"][2]["mixer"]
+    a, d = m2["left"], m2["right"]
+    assert (s2.mixer, s2.heads, s2.kv_heads, s2.dim, s2.vdim, s2.attn_scale) == (Ly.MIX_ATTN, 6, 6, 16, 16, a["scale"])
+    assert (s2.qk_norm, s2.sink, s2.sink_learned, s2.mask_kind, s2.rot_dims) == (Ly.QK_HEAD_W, 1, True, Ly.MASK_CAUSAL, 0)
+    assert (s2.q_temp_coef, s2.q_temp_every, s2.rel_max, s2.rel_rows, s2.join_scale) == (0.4, 1, 9.0, 8, 0.5)
+    sd = s2.side
+    assert (sd.mixer, sd.heads, sd.kv_heads, sd.dim, sd.vdim, sd.conv) == (Ly.MIX_DELTA, d["heads"], d["kv_heads"], d["dim"],
+                                                                          d["vdim"], d["conv"])
+    assert (sd.decay_rank, sd.gate_rank, sd.gate_act, sd.ff_kind) == (5, 12, Ly.DELTA_GATE_SIGMOID, Ly.FF_NONE)
+    assert (s2.ff_kind, s2.experts, s2.top, s2.groups, s2.groups_keep, s2.shared_ff) == (Ly.FF_MOE, 4, 1, 1, 1, 0)
+    s5 = c.layers[5]
+    assert (s5.router_kind, s5.router_biased, s5.groups, s5.groups_keep, s5.shared_ff, s5.shared_gated, s5.ff_act) == (
+        Ly.ROUTER_SIGMOID_GROUPS, True, 4, 2, 8, True, Ly.ACT_SILU)
+    assert c.layers[3].ff_kind == Ly.FF_NONE and c.layers[3].side is None
+    # rows of the concatenated input projections
+    assert s0.in_rows == 2 * 3 * 16 + 2 * 1 * 24 + 3
+    assert sd.in_rows == 2 * 2 * 24 + 2 * 8 + 12 + 2 + 5
+
+
+def test_lifenex_unknown_names_are_refused():
+    import lifenex_cases as LC
+
+    bad = {**LC.ONLY_SSM, "layers": [{"type": "mamba3", "mixer": LC.ssm(), "mlp": None}]}
+    with pytest.raises(ValueError):
+        Ly.lifenex_config(bad)
+    bad = {**LC.ONLY_DENSE, "layers": [{"type": "mamba2", "mixer": LC.ssm(), "mlp": {"kind": "glu", "ff": 8}}]}
+    with pytest.raises(ValueError):
+        Ly.lifenex_config(bad)
+    with pytest.raises(ValueError):  # a pair's table and ranks are the tensors' own sizes
+        Ly.lifenex_config(LC.ONLY_PAIR)
+
+
+def test_lifenex_pack_concatenates_and_nests_the_second_mixer():
+    import lifenex_cases as LC
+
+    cfg = LC.MIXED
+    t = Ly.lifenex_random_tensors(cfg, seed=3, **LC.sizes(cfg))
+    assert set(t) == set(Ly.lifenex_tensor_shapes(cfg, **LC.sizes(cfg)))
+    for wdt in (M.F32, M.BF16):
+        c = Ly.lifenex_config(cfg, weight_dtype=wdt, shapes={k: v.shape for k, v in t.items()})
+        p = Ly.lifenex_pack(c, t)
+        f = (lambda a: a) if wdt == M.F32 else Ly.bf16_to_f32
+        assert p["head"] is p["embed"] and np.array_equal(p["embed_norm"], t["embed.norm"])
+        d0 = p["layers"][0]
+        assert np.array_equal(f(d0["w_in"]), t["l0.mix.in"]) and np.array_equal(d0["d_skip"], t["l0.mix.D"])
+        assert np.array_equal(d0["conv_b"], t["l0.mix.conv.b"]) and np.array_equal(d0["norm2"], t["l0.norm2"])
+        assert "ls1" not in d0 and "side" not in d0 and "w_gate" not in d0
+        d1 = p["layers"][1]
+        assert np.array_equal(f(d1["w_in"]), np.concatenate([t["l1.mix.left." + n] for n in ("q", "k", "v")]))
+        assert np.array_equal(d1["rel"], t["l1.mix.left.rel"]) and np.array_equal(d1["sink_w"], t["l1.mix.left.sink"])
+        assert np.array_equal(d1["join_w"], t["l1.mix.left.out"]) and np.array_equal(d1["side_join_w"], t["l1.mix.right.out"])
+        assert np.array_equal(d1["router_bias"], t["l1.mlp.correction"]) and d1["shared_sg"].shape == (cfg["width"],)
+        assert np.array_equal(f(d1["w_up"][4]), t["l1.mlp.e4.up"])
+        sd = d1["side"]
+        assert np.array_equal(f(sd["w_in"]), np.concatenate([t["l1.mix.right." + n] for n in ("q", "k", "v", "g1", "b", "a1")]))
+        assert np.array_equal(sd["conv_w"], np.concatenate([t["l1.mix.right." + n + ".conv"] for n in ("q", "k", "v")]))
+        assert np.array_equal(f(sd["w_a2"]), t["l1.mix.right.a2"]) and np.array_equal(f(sd["w_g2"]), t["l1.mix.right.g2"])
+        assert "norm1" not in sd and "norm2" not in p["layers"][3]
+        for l, d in zip(c.layers, p["layers"]):
+            assert set(Ly.packed_shapes(c, l)) == set(d) - {"side"}
+            if l.side is not None:
+                assert set(Ly.packed_shapes(c, l.side, side=True)) == set(d["side"])
+
+
+def test_lifenex_restatement_mechanisms():
+    """The restatement itself: causality; the distance buckets; the temperature's blocks; the sink's
+    share; the router's groups (ranked by their two best, forbidden experts behind every allowed
+    one even when all choice scores are negative), its correction and its weights."""
+    import lifenex_cases as LC
+    import lifenex_ref as LR
+
+    cfg = LC.MIXED
+    w = {k: v.astype(np.float64) for k, v in Ly.lifenex_random_tensors(cfg, seed=4, **LC.sizes(cfg)).items()}
+    a = LC.tokens(cfg, 40, 1)
+    b = list(a)
+    b[30] = (b[30] + 1) % cfg["vocab"]
+    ra, rb = LR.forward(cfg, w, a), LR.forward(cfg, w, b)
+    assert np.array_equal(ra[:30], rb[:30]) and not np.allclose(ra[30], rb[30])
+    assert not np.allclose(ra[39], rb[39])  # and the change is carried on (states, keys)
+    # 8 rows reaching 64 back: exact below 4, then 4 logarithmic rows up to 64, the last row beyond
+    bk = LR.distance_bucket(np.arange(200), 8, 64.0)
+    assert bk[:4].tolist() == [0, 1, 2, 3] and bk[4] == 4 and bk[7] == 4 and bk[8] == 5 and bk[15] == 5 and bk[16] == 6
+    assert bk[31] == 6 and bk[32] == 7 and bk[63] == 7 and bk[64] == 7 and bk[199] == 7 and (np.diff(bk) >= 0).all()
+    tq = LR.query_temperature(np.array([0, 6, 7, 14, 20]), 0.5, 7)
+    assert np.allclose(tq, [1.0, 1.0 + 0.5 * np.log(2), 1.0 + 0.5 * np.log(2), 1.0 + 0.5 * np.log(3), 1.0 + 0.5 * np.log(4)])
+    p = LR.softmax_sink(np.array([[0.0, 0.0, -np.inf]]), np.log(2.0))
+    assert np.allclose(p, [[0.25, 0.25, 0.0]])
+    # two groups of three: group 1 wins by the sum of its two best although group 0 holds the best expert
+    z = np.array([3.0, -9.0, -9.0, 2.0, 2.0, -9.0])
+    idx, wt = LR.route(z, np.zeros(6), 2, 2, 1)
+    assert sorted(idx.tolist()) == [3, 4] and np.allclose(wt, LR.sigmoid(2.0))
+    # the correction moves the choice, not the weights; negative choice scores keep forbidden experts out
+    idx, wt = LR.route(z, np.array([0.0, 0.0, 0.0, 0.0, -5.0, 1.2]) - 10.0, 2, 2, 1)
+    assert idx.tolist() == [5, 3] and np.allclose(wt, [LR.sigmoid(-9.0), LR.sigmoid(2.0)])
+    g = LR.grouped_rms(np.array([[3.0, 4.0, 0.0, 5.0]]), 2, np.ones(4), 0.0)
+    assert np.allclose(g, [[3 / np.sqrt(12.5), 4 / np.sqrt(12.5), 0.0, np.sqrt(2.0)]])
+    y = LR.causal_conv(np.array([[1.0], [2.0], [3.0]]), np.array([[10.0, 1.0]]), np.array([0.5]))
+    assert np.allclose(y[:, 0], [1.5, 12.5, 23.5])
