@@ -79,7 +79,7 @@ def parse():
                          "(Sinulorn-shaped stacks, random bf16 weights) at a few real layer sizes, each beside a "
                          "Llama-shaped decoder of equal width, depth and feed-forward size; one JSON line")
     ap.add_argument("--layered-sizes", default="1024,2048,4096", help="model widths of the --layered legs")
-    ap.add_argument("--layered-design", default="sinulorn", choices=["sinulorn", "lenuzen", "mirorax"],
+    ap.add_argument("--layered-design", default="sinulorn", choices=["sinulorn", "lenuzen", "mirorax", "lifenex"],
                     help="which layer-list design the --layered stack is shaped like")
     return ap.parse_args()
 
@@ -578,6 +578,38 @@ def mirorax_stack(Ly, M, width, max_tokens):
                             block_kind=Ly.BLOCK_PARALLEL)
 
 
+def lifenex_stack(Ly, M, width, max_tokens):
+    """A Lifenex-shaped stack at a real layer size, six layers: state-space + relu^2 dense, two
+    pairs (biased attention beside a delta rule with per-channel decays) + routed experts,
+    state-space + experts, pair + dense, pair + experts. State-space heads of 64 channels with a
+    state of 128 rows and 8 B / C groups; attention heads of 128 with four query heads per
+    key/value head, a 32-row distance table reaching 1024 positions back, temperature blocks of
+    512; delta heads of 128 x 128 with rank-64 decay and gate projections; dense hidden size
+    3.5 x width, experts whose active hidden size (top x expert + shared) equals it."""
+    heads = width // 128
+    ff = width * 7 // 2
+    dense = dict(ff_kind=Ly.FF_PLAIN, ff=ff, ff_act=Ly.ACT_RELU2)
+    moe = dict(ff_kind=Ly.FF_MOE, ff=ff // 8, experts=16, top=4, groups=4, groups_keep=2, shared_ff=ff // 2,
+               shared_gated=True, ff_act=Ly.ACT_SILU, router_kind=Ly.ROUTER_SIGMOID_GROUPS, router_biased=True)
+    both = dict(ff_normed=True, layer_scaled=False)
+    ssm = dict(heads=width // 64, vdim=64, ssm_state=128, ssm_groups=8, norm_groups=8, conv=4, **both)
+    att = dict(heads=heads, kv_heads=max(heads // 4, 1), dim=128, vdim=128, attn_scale=128 ** -0.5,
+               mask_kind=Ly.MASK_CAUSAL, qk_norm=Ly.QK_HEAD_W, sink=1, sink_learned=True, q_temp_coef=0.25,
+               q_temp_every=512, rel_rows=32, rel_max=1024.0, join_scale=0.5, **both)
+    L = Ly.LayerSpec
+
+    def pair(**f):
+        side = L(Ly.MIX_DELTA, heads=max(heads // 2, 1), kv_heads=max(heads // 4, 1), dim=128, vdim=128, conv=4,
+                 decay_rank=64, gate_rank=64, gate_act=Ly.DELTA_GATE_SIGMOID)
+        return L(Ly.MIX_ATTN, side=side, **att, **f)
+
+    layers = [L(Ly.MIX_SSM, **ssm, **dense), pair(**moe), pair(**moe), L(Ly.MIX_SSM, **ssm, **moe), pair(**dense),
+              pair(**moe)]
+    return Ly.LayeredConfig("Lifenex", width, 32000, layers, embed_scale=1.0, norm_eps=1e-6, max_tokens=max_tokens,
+                            weight_dtype=M.BF16, norm_kind=Ly.NORM_RMS, pre_norm=True, pos_embed=False,
+                            logit_scale=0.25, tied_head=True, block_kind=Ly.BLOCK_PARALLEL, embed_normed=True)
+
+
 def layered_bench(args, out_file):
     """--layered: tokens/s of a prompt portion (n = 2048 at position 0) and of single-token
     decoding (the device greedy loop at context ~1024) for the layer-list engine, and for a
@@ -591,22 +623,34 @@ def layered_bench(args, out_file):
     n_pf, ctx, steps = 2048, 1024, max(args.steps if args.steps != 256 else 64, 8)
     legs = []
     for width in [int(x) for x in args.layered_sizes.split(",")]:
-        make = {"lenuzen": lenuzen_stack, "mirorax": mirorax_stack}.get(args.layered_design, layered_stack)
+        make = {"lenuzen": lenuzen_stack, "mirorax": mirorax_stack, "lifenex": lifenex_stack}.get(args.layered_design,
+                                                                                                   layered_stack)
+
+        def timed(cfg):
+            model = runtime.SeqModel.synthetic(cfg, seed=3)
+            dec = runtime.SeqDecoder(model)
+            pf_ms = dec.time_step(n_pf, 0, max(args.prefill_iters, 1))
+            dec.reset()
+            dec.step([(7 * i + 1) % cfg.vocab for i in range(ctx)])
+            tok = dec.generate_greedy(1, args.warmup or 1)[-1]
+            t0 = time.perf_counter()
+            dec.generate_greedy(tok, steps)
+            dt = time.perf_counter() - t0
+            dec.close()
+            model.close()
+            return pf_ms, dt
+
         cfg = make(Ly, M, width, n_pf + 64)
-        model = runtime.SeqModel.synthetic(cfg, seed=3)
-        dec = runtime.SeqDecoder(model)
-        pf_ms = dec.time_step(n_pf, 0, max(args.prefill_iters, 1))
-        dec.reset()
-        dec.step([(7 * i + 1) % cfg.vocab for i in range(ctx)])
-        tok = dec.generate_greedy(1, args.warmup or 1)[-1]
-        t0 = time.perf_counter()
-        dec.generate_greedy(tok, steps)
-        dt = time.perf_counter() - t0
+        pf_ms, dt = timed(cfg)
         leg = {"width": width, "layers": len(cfg.layers), "prefill_tokens": n_pf, "prefill_ms": round(pf_ms, 3),
                "prefill_tok_s": round(n_pf / pf_ms * 1e3, 1), "decode_context": ctx, "decode_steps": steps,
                "decode_ms_per_token": round(dt / steps * 1e3, 4), "decode_tok_s": round(steps / dt, 2)}
-        dec.close()
-        model.close()
+        if args.layered_design == "lifenex":
+            # the closest layer-list design (delta rule, a linear recurrence, grouped routed experts with a
+            # gated shared expert, attention) at the same width, depth and feed-forward size
+            npf, ndt = timed(layered_stack(Ly, M, width, n_pf + 64))
+            leg.update(near_design="Sinulorn", near_prefill_ms=round(npf, 3), near_prefill_tok_s=round(n_pf / npf * 1e3, 1),
+                       near_decode_ms_per_token=round(ndt / steps * 1e3, 4), near_decode_tok_s=round(steps / ndt, 2))
         ref = M.ModelConfig(dim=width, hidden_dim=width * 7 // 2, head_dim=128, n_layers=len(cfg.layers),
                             n_heads=width // 128, n_kv_heads=max(width // 512, 1), vocab_size=32000,
                             max_seq_len=n_pf + 64, weight_dtype=M.F16)
