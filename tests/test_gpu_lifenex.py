@@ -145,6 +145,40 @@ def test_each_mixer_of_a_pair_alone(rt, which):
         model.close()
 
 
+def test_pair_in_serial_blocks(rt):
+    """Two mixers side by side are a mechanism of the engine, not of one design: the same pair in
+    the OTHER envelope (serial blocks, a closing norm after the sublayer), put together by hand;
+    the join is then a launch of its own instead of a part of the parallel block's seam."""
+    from yalm_amd import layered as Ly
+    from yalm_amd import models as M
+
+    cfg = C.ONLY_PAIR
+    t = make(cfg, 33)
+    w = {k: v.astype(np.float64) for k, v in t.items()}
+    c = Ly.lifenex_config(cfg, max_tokens=256, weight_dtype=M.F32, shapes={k: v.shape for k, v in t.items()})
+    p = Ly.lifenex_pack(c, t)
+    closing = (1.0 + 0.1 * np.arange(cfg["width"]) / cfg["width"]).astype(np.float32)
+    spec = dataclasses.replace(c.layers[0], ff_normed=False)
+    c1 = c.with_(layers=[spec], block_kind=Ly.BLOCK_SERIAL)
+    pd = dict(p["layers"][0], norm1b=closing)
+    assert set(pd) - {"side"} == set(Ly.packed_shapes(c1, spec))
+    model = rt.SeqModel.from_packed(c1, dict(p, layers=[pd]))
+    dec = rt.SeqDecoder(model)
+    try:
+        tok = C.tokens(cfg, 80, 33)
+        eps = cfg["norm"]["eps"]
+        x = R.rms_norm(w["embed"][tok], w["embed.norm"], eps)
+        y = R.mixer_pair(cfg, w, "l0.mix.", R.rms_norm(x, w["l0.norm1"], eps), cfg["layers"][0]["mixer"])
+        x = x + R.rms_norm(y, closing.astype(np.float64), eps)
+        ref = R.rms_norm(x, w["final.norm"], eps) @ w["embed"].T * cfg["logit_scale"]
+        for sizes in ([80], [30] + [1] * 50, [2, 9, 3, 8, 33]):
+            dec.reset()
+            assert rel_err(run_portions(dec, tok, sizes), ref).max() < F32_TOL
+    finally:
+        dec.close()
+        model.close()
+
+
 @pytest.mark.parametrize("name", ["mixed", "odd", "wide", "dense_only"])
 def test_residual_stream_after_every_layer(rt, name):
     from yalm_amd import models as M

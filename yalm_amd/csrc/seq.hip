@@ -810,24 +810,25 @@ static int mixer_rglru(Seq *q, int li, int n) {
 // and key channel) or the state-space walk (ssm = true). K: key / state size, P: value size.
 static int delta_launch(Seq *q, const float *qkv, int ldq, int qo, int ko, int vo, int KH, int K, int H, int P,
                         const float *bg, const float *gv, const float *dskip, float *state, float *o, int n, bool ssm) {
-	const dim3 g(cdiv(P, SEQ_THREADS / 8), H);
-	const int R = cdiv(K, 8);
-#define DELTA_LAUNCH(RR, TC)                                                                                           \
+	// lanes per column of the state: 16 (twice the workgroups, half the rows per lane) but for the smallest keys
+	const int lpc = K <= 32 ? 8 : 16;
+	const dim3 g(cdiv(P, SEQ_THREADS / lpc), H);
+#define DELTA_LAUNCH(RR, TC, LPC)                                                                                      \
 	do {                                                                                                               \
 		if (ssm)                                                                                                       \
-			seq_delta_kernel<RR, TC, true, false><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, ldq, qo, ko, vo, KH, K, H, P, bg, \
-			                                                                        nullptr, dskip, state, o, n);          \
+			seq_delta_kernel<RR, TC, true, false, LPC><<<g, SEQ_THREADS, 0, q->stream>>>(                              \
+			    qkv, ldq, qo, ko, vo, KH, K, H, P, bg, nullptr, dskip, state, o, n);                                   \
 		else if (gv)                                                                                                   \
-			seq_delta_kernel<RR, TC, false, true><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, ldq, qo, ko, vo, KH, K, H, P, bg, \
-			                                                                        gv, nullptr, state, o, n);             \
+			seq_delta_kernel<RR, TC, false, true, LPC><<<g, SEQ_THREADS, 0, q->stream>>>(                              \
+			    qkv, ldq, qo, ko, vo, KH, K, H, P, bg, gv, nullptr, state, o, n);                                      \
 		else                                                                                                           \
-			seq_delta_kernel<RR, TC, false, false><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, ldq, qo, ko, vo, KH, K, H, P,   \
-			                                                                         bg, nullptr, nullptr, state, o, n);   \
+			seq_delta_kernel<RR, TC, false, false, LPC><<<g, SEQ_THREADS, 0, q->stream>>>(                             \
+			    qkv, ldq, qo, ko, vo, KH, K, H, P, bg, nullptr, nullptr, state, o, n);                                 \
 	} while (0)
-	if (R <= 4) DELTA_LAUNCH(4, 16);
-	else if (R <= 8) DELTA_LAUNCH(8, 16);
-	else if (R <= 16) DELTA_LAUNCH(16, 16);
-	else DELTA_LAUNCH(32, 8);
+	if (K <= 32) DELTA_LAUNCH(4, 16, 8);
+	else if (K <= 64) DELTA_LAUNCH(4, 16, 16);
+	else if (K <= 128) DELTA_LAUNCH(8, 16, 16);
+	else DELTA_LAUNCH(16, 8, 16);
 #undef DELTA_LAUNCH
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
@@ -1340,12 +1341,14 @@ static int par_close(Seq *q, int li, int n) {
 	const yalm_seq_layer *nx = li + 1 < c.n_layers ? &q->L[li + 1] : nullptr;
 	const bool moe = l.ff_kind == YALM_FF_MOE;
 	const bool gated = moe && l.shared_ff > 0 && l.shared_sg;
+	const bool joined = q->side_of[li] >= 0; // two mixers side by side: their normed results meet in this launch
 	float *dump = q->dump_on && q->dump ? q->dump + (size_t)li * n * c.width : nullptr;
 #define PC_ARGS                                                                                                        \
 	q->X, q->Y, l.ls1, (l.ff_kind != YALM_FF_NONE && !moe) ? q->Y2 : nullptr, l.ls2, moe ? q->B[1] : nullptr, q->wt,    \
 	    moe ? l.top : 0, moe && l.shared_ff > 0 ? q->B[3] : nullptr, gated ? q->sgate : nullptr, dump,                 \
 	    nx ? nx->pre_add : nullptr, c.norm_eps, c.width, nx ? nx->norm1 : nullptr, q->Hn, (int)q->ln,                  \
-	    (nx && nx->ff_kind != YALM_FF_NONE) ? nx->norm2 : nullptr, q->Hn2
+	    (nx && nx->ff_kind != YALM_FF_NONE) ? nx->norm2 : nullptr, q->Hn2, joined ? q->Y3 : nullptr, l.join_w,        \
+	    l.side_join_w, l.join_scale
 	if (c.width <= 4 * SEQ_THREADS)
 		seq_par_close_reg_kernel<4><<<n, SEQ_THREADS, 0, q->stream>>>(PC_ARGS);
 	else if (c.width <= 8 * SEQ_THREADS)
@@ -1440,9 +1443,11 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 			const int rc = run_mixer(side);
 			q->Yout = q->Y;
 			TRY(rc);
-			seq_pair_join_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(q->Y, q->Y3, l.join_w, l.side_join_w, l.join_scale,
-			                                                       c.norm_eps, c.width);
-			HIPCHK(hipGetLastError());
+			if (!par) { // serial blocks: joined here; a parallel block's seam joins them itself
+				seq_pair_join_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(q->Y, q->Y3, l.join_w, l.side_join_w, l.join_scale,
+				                                                       c.norm_eps, c.width);
+				HIPCHK(hipGetLastError());
+			}
 		}
 		if (par) { // both sublayers read norms of the same stream; the feed-forward's result goes beside the mixer's
 			const float *mix_in = q->In;

@@ -352,7 +352,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__rest
 // the row after the sums is also written there (the stream as the block leaves it). Then
 // X[t] += add (the vector the next layer adds before its opening norm) and, if w_next, Hn[t]
 // = norm(X[t]) * w_next and, with w_next2, Hn2[t] = norm(X[t]) * w_next2 (the norm the next
-// block's feed-forward reads). s1 / s2 == nullptr: scale 1. Dynamic LDS: n floats.
+// block's feed-forward reads). s1 / s2 == nullptr: scale 1. Yb != nullptr: the block has two
+// mixers side by side and its mixer row is jscale (rms(Y1[t]) ja + rms(Yb[t]) jb), each row
+// divided by its own root mean square over n (no mean taken off). Dynamic LDS: n floats.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__restrict__ X, const float *__restrict__ Y1,
                                                                     const float *__restrict__ s1,
                                                                     const float *__restrict__ Y2,
@@ -366,14 +368,32 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_kernel(float *__res
                                                                     const float *__restrict__ w_next,
                                                                     float *__restrict__ Hn, int ln,
                                                                     const float *__restrict__ w_next2 = nullptr,
-                                                                    float *__restrict__ Hn2 = nullptr) {
+                                                                    float *__restrict__ Hn2 = nullptr,
+                                                                    const float *__restrict__ Yb = nullptr,
+                                                                    const float *__restrict__ ja = nullptr,
+                                                                    const float *__restrict__ jb = nullptr,
+                                                                    float jscale = 1.0f) {
 	extern __shared__ float row[];
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	float *x = X + (size_t)t * n;
+	float ra = 1.0f, rb = 0.0f;
+	if (Yb) {
+		float sa = 0.0f, sb = 0.0f;
+		for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+			const float a = Y1[(size_t)t * n + i], b = Yb[(size_t)t * n + i];
+			sa = fmaf(a, a, sa);
+			sb = fmaf(b, b, sb);
+		}
+		ra = jscale / sqrtf(block_sum(sa, red) / (float)n + eps);
+		rb = jscale / sqrtf(block_sum(sb, red) / (float)n + eps);
+	}
 	float ss = 0.0f, sm = 0.0f;
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
-		float v = fmaf(s1 ? s1[i] : 1.0f, Y1[(size_t)t * n + i], x[i]);
+		float y1 = Y1[(size_t)t * n + i];
+		if (Yb)
+			y1 = y1 * ra * ja[i] + Yb[(size_t)t * n + i] * rb * jb[i];
+		float v = fmaf(s1 ? s1[i] : 1.0f, y1, x[i]);
 		if (Yx) {
 			float f = 0.0f;
 			for (int k = 0; k < top; ++k)
@@ -430,7 +450,11 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_reg_kernel(float *_
                                                                         const float *__restrict__ w_next,
                                                                         float *__restrict__ Hn, int ln,
                                                                         const float *__restrict__ w_next2 = nullptr,
-                                                                        float *__restrict__ Hn2 = nullptr) {
+                                                                        float *__restrict__ Hn2 = nullptr,
+                                                                        const float *__restrict__ Yb = nullptr,
+                                                                        const float *__restrict__ ja = nullptr,
+                                                                        const float *__restrict__ jb = nullptr,
+                                                                        float jscale = 1.0f) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	float x[E], y1[E], a1[E], f[E], a2[E], ad[E], wn[E];
@@ -446,6 +470,24 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_par_close_reg_kernel(float *_
 		ad[e] = (in && add) ? add[i] : 0.0f;
 		wn[e] = (in && w_next) ? w_next[i] : 0.0f;
 		f[e] = (in && Y2 && !Yx) ? Y2[(size_t)t * n + i] : 0.0f;
+	}
+	if (Yb) { // two mixers side by side: the normed rows joined before anything else reads y1
+		float yb[E], sa = 0.0f, sb = 0.0f;
+#pragma unroll
+		for (int e = 0; e < E; ++e) {
+			const int i = threadIdx.x + e * SEQ_THREADS;
+			yb[e] = i < n ? Yb[(size_t)t * n + i] : 0.0f;
+			sa = fmaf(y1[e], y1[e], sa);
+			sb = fmaf(yb[e], yb[e], sb);
+		}
+		const float ra = jscale / sqrtf(block_sum(sa, red) / (float)n + eps);
+		const float rb = jscale / sqrtf(block_sum(sb, red) / (float)n + eps);
+#pragma unroll
+		for (int e = 0; e < E; ++e) {
+			const int i = threadIdx.x + e * SEQ_THREADS;
+			if (i < n)
+				y1[e] = y1[e] * ra * ja[i] + yb[e] * rb * jb[i];
+		}
 	}
 	if (Yx) {
 		for (int k = 0; k < top; ++k) {
@@ -1398,19 +1440,28 @@ __device__ __forceinline__ float sum8(float v) { // over aligned groups of 8 lan
 	v += dpp<0x141>(v);
 	return v;
 }
+template <int LPC>
+__device__ __forceinline__ float sum_lanes(float v) { // over aligned groups of LPC = 8 or 16 lanes
+	v = sum8(v);
+	if constexpr (LPC == 16)
+		v += dpp<0x140>(v);
+	return v;
+}
 
 // The recurrence itself. The columns of a head's [dim][vdim] state never mix, so one group
-// of 8 lanes owns one column (each lane a contiguous slice of R dim entries, in registers)
-// and walks the portion's tokens in order:
+// of LPC (8 or 16) lanes owns one column (each lane a contiguous slice of R dim entries, in
+// registers; LPC R >= dim) and walks the portion's tokens in order:
 //   S *= g;  u = beta (v - S.k);  S += k u;  o = S.q
-// (the read-out after the write). The workgroup's 32 columns share the head's k and q:
+// (the read-out after the write). The workgroup's 256 / LPC columns share the head's k and q:
 // chunks of TC tokens are staged through two LDS buffers, the next chunk's global loads in
-// flight while the current chunk is applied. grid (ceil(vdim / 32), heads).
+// flight while the current chunk is applied. grid (ceil(vdim LPC / 256), heads). 16 lanes per
+// column halve every lane's rows (a shorter dependent chain and half the LDS reads per token)
+// and double the workgroups of a walk that fills a fraction of the chip.
 // SSM: the state-space form of the same walk, S *= g; S += k (beta v); o = S.q + dskip[h] v
 // (no prediction S.k is taken off the write; k, q, v, beta are the layer's B, C, x and dt).
 // GVEC: g is a vector over the key channels, GV [T][H D], instead of one number per head.
 // QKV [T][ldq]: key/query head kh's q at column qo + kh D, its k at ko + kh D, head h's v at vo + h V.
-template <int R, int TC, bool SSM, bool GVEC>
+template <int R, int TC, bool SSM, bool GVEC, int LPC>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__restrict__ QKV, int ldq, int qo_, int ko_,
                                                                 int vo_, int KH, int D, int H, int V,
                                                                 const float *__restrict__ BG,
@@ -1418,15 +1469,16 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
                                                                 const float *__restrict__ dskip,
                                                                 float *__restrict__ state, float *__restrict__ O,
                                                                 int T) {
-	constexpr int DP = 8 * R;                      // padded key dimension
+	constexpr int DP = LPC * R;                    // padded key dimension
 	constexpr int NS = GVEC ? 3 : 2;               // staged rows per token: k | q (| g)
 	constexpr int NKQ = TC * NS * DP / SEQ_THREADS; // staged values per thread and chunk
-	constexpr int COLS = SEQ_THREADS / 8, NV = (TC * COLS + SEQ_THREADS - 1) / SEQ_THREADS;
+	constexpr int COLS = SEQ_THREADS / LPC, NV = (TC * COLS + SEQ_THREADS - 1) / SEQ_THREADS;
+	static_assert((LPC == 8 || LPC == 16) && (TC * NS * DP) % SEQ_THREADS == 0, "staging assumes whole passes of the workgroup");
 	__shared__ __attribute__((aligned(16))) float kq[2][TC][NS * DP];
 	__shared__ float vs[2][TC][COLS], bgs[2][TC][2];
 	const int tid = threadIdx.x;
 	const int h = blockIdx.y, kh = h / (H / KH);
-	const int c0 = blockIdx.x * COLS, col = c0 + (tid >> 3), sub = tid & 7;
+	const int c0 = blockIdx.x * COLS, col = c0 + tid / LPC, sub = tid % LPC;
 	const bool live = col < V;
 	const int d0 = sub * R; // this lane's slice of the key dimension: d0 .. d0 + R - 1
 	float S[R];
@@ -1521,7 +1573,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 						x.gv[i] = kq[buf][tt][2 * DP + d0 + i];
 				}
 			}
-			x.v = vs[buf][tt][tid >> 3];
+			x.v = vs[buf][tt][tid / LPC];
 			x.beta = bgs[buf][tt][0];
 			x.g = bgs[buf][tt][1];
 		};
@@ -1544,7 +1596,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 			if constexpr (SSM)
 				u = x.beta * x.v;
 			else
-				u = x.beta * (x.v - sum8(dd0 + dd1));
+				u = x.beta * (x.v - sum_lanes<LPC>(dd0 + dd1));
 			float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
 			for (int i = 0; i < R; ++i) {
@@ -1554,7 +1606,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 				else
 					o0 = fmaf(S[i], x.q[i], o0);
 			}
-			float o = sum8(o0 + o1);
+			float o = sum_lanes<LPC>(o0 + o1);
 			if constexpr (SSM)
 				o = fmaf(dsk, x.v, o);
 			if (sub == 0 && live)
