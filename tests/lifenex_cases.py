@@ -80,7 +80,7 @@ ODD = config([
     (P, pair(attn(heads=2, kv_heads=1, dim=9, vdim=7, scale=0.5, bias_max=33, every=5),
              delta(heads=2, kv_heads=2, dim=7, vdim=5, conv=1)), None),
     (S, ssm(heads=1, vdim=13, state=11, groups=1, norm_groups=1, conv=2), moe(experts=6, top=2, ff=9, shared=0, count=2, keep=1)),
-], width=50, vocab=37, eps=1e-4, logit_scale=1.7, sizes={"rel_rows": 6, "decay_rank": 3, "gate_rank": 1})
+], width=50, vocab=37, eps=1e-4, logit_scale=1.7, sizes={"rel_rows": 7, "decay_rank": 3, "gate_rank": 1})
 # wider sizes: several tiles per product, key rows and states of more than 64 entries, many heads
 WIDE = config([
     (S, ssm(heads=8, vdim=64, state=128, groups=2, norm_groups=4, conv=4), dense(ff=320)),

@@ -1016,6 +1016,13 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 		const bool need = wave_on && kt <= whi && kt + SAM_KT - 1 >= wlo;
 		if (need) {
 			f32x4a_t sacc[2] = {f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f}};
+			// the distance biases of this lane's eight scores: loaded now, in flight under the products
+			float rb0[4], rb1[4];
+#pragma unroll
+			for (int r = 0; r < 4; ++r) {
+				rb0[r] = attn_rel_bias(a, h, hi_[r] - (kt + lr));
+				rb1[r] = attn_rel_bias(a, h, hi_[r] - (kt + 16 + lr));
+			}
 #pragma unroll
 			for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
@@ -1030,8 +1037,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 			for (int r = 0; r < 4; ++r) {
 				const int j0 = kt + lr, j1 = kt + 16 + lr;
 				const bool v0 = j0 >= lo_[r] && j0 <= hi_[r], v1 = j1 >= lo_[r] && j1 <= hi_[r];
-				const float s0 = v0 ? sacc[0][r] + attn_rel_bias(a, h, hi_[r] - j0) : -FLT_MAX;
-				const float s1 = v1 ? sacc[1][r] + attn_rel_bias(a, h, hi_[r] - j1) : -FLT_MAX;
+				const float s0 = v0 ? sacc[0][r] + rb0[r] : -FLT_MAX;
+				const float s1 = v1 ? sacc[1][r] + rb1[r] : -FLT_MAX;
 				const float mnew = fmaxf(mrun[r], row16_max(fmaxf(s0, s1)));
 				const float p0 = v0 ? expf(s0 - mnew) : 0.0f, p1 = v1 ? expf(s1 - mnew) : 0.0f;
 				al[r] = expf(mrun[r] - mnew);
