@@ -630,6 +630,25 @@ def test_large_head_sizes(rt, name):
             model.close()
 
 
+def test_stream_wider_than_the_register_seam(rt):
+    """A width above 4096 takes the seam kernel that keeps the row in LDS (join of the pair, experts'
+    combine, both opening norms) and the embedding / norm kernels' strided loops."""
+    from yalm_amd import models as M
+
+    cfg = C.config([(C.P, C.pair(C.attn(heads=2, kv_heads=1, dim=16, vdim=8, scale=0.25, bias_max=20, every=8),
+                                 C.delta(heads=2, kv_heads=1, dim=8, vdim=8, conv=2)), C.moe(experts=4, top=2, ff=8, shared=8, count=2, keep=1)),
+                    (C.S, C.ssm(heads=2, vdim=8, state=8, groups=1, norm_groups=2, conv=2), C.dense(ff=16))],
+                   width=4104, vocab=41, sizes={"rel_rows": 6, "decay_rank": 2, "gate_rank": 2})
+    model, dec, w = build(rt, cfg, M.F32, seed=23, max_tokens=64)
+    try:
+        tok = C.tokens(cfg, 40, 23)
+        ref = R.forward(cfg, w, tok)
+        assert rel_err(run_portions(dec, tok, [12, 3, 9] + [1] * 16), ref).max() < F32_TOL
+    finally:
+        dec.close()
+        model.close()
+
+
 def test_sequence_cannot_pass_max_tokens(rt):
     from yalm_amd import models as M
 
